@@ -1,0 +1,119 @@
+"""ctypes binding of the gfx950 shared library (C ABI declared in ``include/chill_attention.h``).
+
+The library is the only compute path: if it has not been built, importing this module raises, and
+nothing in the package falls back to another implementation.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_uint8, c_void_p
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libchill_attention_hip.so")
+
+ABI_VERSION = 1
+
+# ChillDType / ChillMaskId / ChillPass of the header
+F32, F16, BF16 = 0, 1, 2
+MASK_FULL, MASK_CAUSAL, MASK_SLIDING_WINDOW, MASK_CHUNKWISE, MASK_PREFIX_LM = range(5)
+PASS_FWD, PASS_DQ, PASS_DKDV = 0, 1, 2
+
+
+class ChillMaskDesc(ctypes.Structure):
+    _fields_ = [("id", c_int32), ("nargs", c_int32), ("args", c_int64 * 4)]
+
+
+class ChillTensor4(ctypes.Structure):
+    _fields_ = [("ptr", c_void_p), ("stride", c_int64 * 4)]
+
+
+class ChillLibraryError(RuntimeError):
+    """A C-ABI call returned a negative status."""
+
+    def __init__(self, fn: str, status: int, text: str):
+        super().__init__(f"{fn} failed with status {status}: {text}")
+        self.status = status
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"chill_attention: the HIP library {LIB_PATH} has not been built "
+            "(run `make -C chill-attention_amd/csrc -j8` or `python -c 'import __graft_entry__ as g; g.build()'`). "
+            "There is no fallback implementation."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    P = POINTER
+    T4 = P(ChillTensor4)
+    MD = P(ChillMaskDesc)
+    I64_3 = P(c_int64)
+    sig = {
+        "chill_fwd": (c_int32, [T4, T4, T4, T4, c_void_p, I64_3, c_void_p, c_int64,
+                                c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
+        "chill_bwd_delta": (c_int32, [T4, T4, c_void_p, I64_3, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p]),
+        "chill_bwd_dq": (c_int32, [T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, I64_3, c_void_p, c_int64,
+                                   c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
+        "chill_bwd_dkdv": (c_int32, [T4, T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, I64_3, c_void_p, c_int64,
+                                     c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
+        "chill_mask_eval_device": (c_int32, [MD, c_int32, c_void_p, c_void_p]),
+        "chill_tile_ranges_device": (c_int32, [MD, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
+        "chill_mask_eval": (c_int32, [MD, c_int32, P(c_uint8)]),
+        "chill_mask_limits": (c_int32, [MD, c_int32, c_int32, c_int32, P(c_int32)]),
+        "chill_tile_ranges": (c_int32, [MD, c_int32, c_int32, c_int32, c_int32, c_int32, P(c_int32)]),
+        "chill_mask_is_full_block": (c_int32, [MD, c_int32, c_int32, c_int32, c_int32, c_int32]),
+        "chill_mask_has_full_blocks": (c_int32, [MD, c_int32, c_int32, c_int32]),
+        "chill_tile_config": (c_int32, [c_int32, c_int32, c_int32, c_int32, P(c_int32)]),
+        "chill_mask_nnz": (c_int64, [MD, c_int32]),
+        "chill_status_string": (c_char_p, [c_int32]),
+        "chill_abi_version": (c_int32, []),
+    }
+    for name, (restype, argtypes) in sig.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype = restype
+        fn.argtypes = argtypes
+    got = lib.chill_abi_version()
+    if got != ABI_VERSION:
+        raise ImportError(f"chill_attention: library ABI version {got}, binding expects {ABI_VERSION}")
+    return lib
+
+
+lib = _load()
+EXPORTED_SYMBOLS = (
+    "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dkdv", "chill_mask_eval_device",
+    "chill_tile_ranges_device", "chill_mask_eval", "chill_mask_limits", "chill_tile_ranges",
+    "chill_mask_is_full_block", "chill_mask_has_full_blocks", "chill_tile_config", "chill_mask_nnz",
+    "chill_status_string", "chill_abi_version",
+)
+
+
+def check(fn: str, status: int) -> int:
+    """Raise for a negative status, pass non-negative values through."""
+    if status < 0:
+        raise ChillLibraryError(fn, status, lib.chill_status_string(status).decode())
+    return status
+
+
+def mask_desc(mask_id: int, args) -> ChillMaskDesc:
+    d = ChillMaskDesc()
+    d.id = mask_id
+    d.nargs = len(args)
+    if len(args) > 4:
+        raise ValueError("a mask descriptor carries at most 4 arguments")
+    for i, a in enumerate(args):
+        d.args[i] = int(a)
+    return d
+
+
+def tensor4(t) -> ChillTensor4:
+    """View of a 4-d torch tensor: raw pointer + element strides."""
+    v = ChillTensor4()
+    v.ptr = t.data_ptr()
+    for i in range(4):
+        v.stride[i] = t.stride(i)
+    return v
+
+
+def strides3(t):
+    return (c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))

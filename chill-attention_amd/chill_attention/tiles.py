@@ -1,0 +1,48 @@
+"""Static MI355X tile table (the counterpart of the reference's ``autotune.py`` default tables).
+
+The table itself is compiled into the HIP library (``csrc/chill_tiles.h``) so the kernels and this
+report cannot disagree; these helpers only read it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+
+_DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
+
+
+def tile_config(mask, head_dim: int, dtype: torch.dtype, pass_id: int) -> dict:
+    """Tile shape the library uses for ``(mask class, head_dim, dtype, pass)``.
+
+    Returns ``{"rows", "streamed", "waves", "lds_bytes"}``: resident rows per workgroup (query
+    rows for forward / dQ, key rows for dK/dV), rows of one streamed tile, wavefronts per
+    workgroup and LDS bytes per workgroup.
+    """
+    out = (ctypes.c_int32 * 4)()
+    _lib.check(
+        "chill_tile_config",
+        _lib.lib.chill_tile_config(mask.mask_id, head_dim, _DTYPES[dtype], pass_id, out),
+    )
+    return {"rows": out[0], "streamed": out[1], "waves": out[2], "lds_bytes": out[3]}
+
+
+def _get_default_config_fwd(head_dim, dtype, mask=None):
+    """(TILE_Q, TILE_K, waves) of the forward kernel — cf. reference autotune.py:98-107."""
+    from .mask import CausalChillMask
+
+    c = tile_config(mask or CausalChillMask(), head_dim, dtype, _lib.PASS_FWD)
+    return c["rows"], c["streamed"], c["waves"]
+
+
+def _get_default_config_bwd(head_dim, dtype, mask=None):
+    """((TILE_DQ_Q, TILE_DQ_K, waves), (TILE_DK_Q, TILE_DK_K, waves)) — cf. reference autotune.py:110-119."""
+    from .mask import CausalChillMask
+
+    m = mask or CausalChillMask()
+    dq = tile_config(m, head_dim, dtype, _lib.PASS_DQ)
+    dk = tile_config(m, head_dim, dtype, _lib.PASS_DKDV)
+    return (dq["rows"], dq["streamed"], dq["waves"]), (dk["streamed"], dk["rows"], dk["waves"])

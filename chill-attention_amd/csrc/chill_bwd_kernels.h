@@ -1,0 +1,411 @@
+// Backward kernels: delta = rowsum(O * dO), dQ, and dK/dV — the gfx950 counterparts of the
+// reference's _chill_attn_bwd_precompute (chill_attention/utils.py:94-217), _chill_attn_bwd_dq
+// (chill_bwd_dq.py:15-397) and _chill_attn_bwd_dkdv (chill_bwd_dkdv.py:15-509).
+//
+// Both matrix kernels use the building blocks of the forward: a wave owns 32 resident rows whose
+// operands sit in registers as MFMA B operands; the streamed tiles sit in LDS and are read both
+// row-wise (products with the resident rows) and through the transposing read (products that
+// accumulate INTO the resident rows).  All accumulators are transposed ([head dim][resident row]),
+// so every per-row quantity is a per-lane scalar.
+//
+//   dQ   (resident: Q, dO rows; streamed: K, V tiles)
+//        S^T = K Q^T, dP^T = V dO^T, P^T = exp2(S^T * scale - LSE2), dS^T = P^T o (dP^T - delta),
+//        dQ^T += K^T dS^T, finally dQ *= sm_scale                      (chill_bwd_dq.py:312-332, 396)
+//   dKdV (resident: K, V rows; streamed: Q, dO tiles with their LSE2 / delta)
+//        S = Q K^T, dP = dO V^T, P, dS as above,
+//        dV^T += dO^T P, dK^T += Q^T dS, finally dK *= sm_scale        (chill_bwd_dkdv.py:362-403, 230)
+#pragma once
+
+#include "chill_device.h"
+#include "chill_params.h"
+#include "chill_tiles.h"
+
+namespace chill {
+
+// ------------------------------------------------------------------------------------------ delta
+// One 16-byte chunk of O and of dO per thread and step; the CH lanes that share a row reduce with
+// butterfly shuffles.  Pure streaming: 2 * D * es bytes read and 4 bytes written per row.
+template <typename E, int D>
+__global__ __launch_bounds__(256) void delta_kernel(DeltaParams p) {
+    using ET = typename Elem<E>::type;
+    constexpr int CH = LdsTile<E, D>::CH;      // lanes per row (2 .. 64)
+    constexpr int EPC = 16 / Elem<E>::kBytes;  // elements per chunk
+    constexpr int ROWS_PER_STEP = 256 / CH;
+    constexpr int STEPS = 4;
+    const int b = blockIdx.z, hd = blockIdx.y;
+    const ET* obase = reinterpret_cast<const ET*>(p.o) + b * p.so.b + hd * p.so.h;
+    const ET* dobase = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hd * p.sdo.h;
+    float* dbase = p.delta + b * p.delta_b + hd * p.delta_h;
+    const int c = threadIdx.x % CH;
+    const int rsub = threadIdx.x / CH;
+    const int row0 = blockIdx.x * (ROWS_PER_STEP * STEPS);
+    i32x4 ov[STEPS], dv[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        int row = row0 + s * ROWS_PER_STEP + rsub;
+        ov[s] = i32x4{0, 0, 0, 0};
+        dv[s] = i32x4{0, 0, 0, 0};
+        if (row < p.T) {
+            ov[s] = *reinterpret_cast<const i32x4*>(reinterpret_cast<const char*>(obase + (int64_t)row * p.so.t) + c * 16);
+            dv[s] = *reinterpret_cast<const i32x4*>(reinterpret_cast<const char*>(dobase + (int64_t)row * p.sdo.t) + c * 16);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        int row = row0 + s * ROWS_PER_STEP + rsub;
+        const ET* oe = reinterpret_cast<const ET*>(&ov[s]);
+        const ET* de = reinterpret_cast<const ET*>(&dv[s]);
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPC; e++) acc += Elem<E>::to_float(oe[e]) * Elem<E>::to_float(de[e]);
+#pragma unroll
+        for (int off = CH / 2; off >= 1; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (c == 0 && row < p.T) dbase[row] = acc;
+    }
+}
+
+template <typename E, int D>
+int launch_delta(const DeltaParams& p, hipStream_t stream) {
+    constexpr int CH = LdsTile<E, D>::CH;
+    constexpr int ROWS_PER_BLOCK = (256 / CH) * 4;
+    dim3 grid(cdiv(p.T, ROWS_PER_BLOCK), p.H, p.B), block(256);
+    if (p.H > 65535 || p.B > 65535) return CHILL_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((delta_kernel<E, D>), grid, block, 0, stream, p);
+    return hipGetLastError() == hipSuccess ? CHILL_OK : CHILL_ERR_HIP;
+}
+
+// Probabilities and score gradients of one 32x32 block, in place: on entry s = raw scores,
+// dp = dO.V products; on exit s = P (0 where masked), dp = dS = P * (dP - delta).
+// Row/column meaning differs between the two kernels, so the caller supplies, per accumulator
+// register r, the LSE2 / delta of the query and the (q, k) positions.
+template <int MASK, bool PARTIAL, typename PosFn>
+__device__ __forceinline__ void softmax_grad_block(f32x16& s, f32x16& dp, float scale, int seq_len,
+                                                   MaskArgs a, PosFn pos) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        int q, k;
+        float lse, delta;
+        pos(r, q, k, lse, delta);
+        float pv = fast_exp2(s[r] * scale - lse);
+        if (PARTIAL) {
+            bool ok = (q < seq_len) && (k < seq_len) && Mask<MASK>::pred(q, k, seq_len, a);
+            pv = ok ? pv : 0.f;
+        }
+        s[r] = pv;
+        dp[r] = pv * (dp[r] - delta);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ dQ
+template <typename E, int D, int MASK, int NW, int TK>
+__global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
+                                                     int wave_has_full_blocks) {
+    using ET = typename Elem<E>::type;
+    constexpr int TQ = NW * 32;
+    constexpr int NT = NW * 64;
+    constexpr int KB = TK / 32;
+    constexpr int DB = (D + 31) / 32;
+    constexpr int TILE_BYTES = LdsTile<E, D>::bytes(TK);
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    if (item < 0) return;
+    const int bh = item / n_q_tiles;
+    const int qt = n_q_tiles - 1 - item % n_q_tiles;
+    const int b = bh / p.H;
+    const int hd = bh % p.H;
+    const int hkv = hd / p.group;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int n = lane & 31;
+    const int h = lane >> 5;
+
+    int seq_len = p.T;
+    if (p.lens != nullptr) seq_len = imin(p.lens[(int64_t)b * p.lens_stride], p.T);
+
+    const int qb = qt * TQ;
+    ET* dqbase = reinterpret_cast<ET*>(p.dq) + b * p.sdq.b + hd * p.sdq.h;
+    if (qb >= seq_len) {
+        zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(TQ, p.T - qb), tid);
+        return;
+    }
+
+    const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hd * p.sq.h;
+    const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hd * p.sdo.h;
+    const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
+    const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
+
+    const int qw = qb + 32 * wave;
+    const int q_pos = qw + n;
+    Resident<E, D> qf, dof;
+    load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
+    load_resident<E, D>(dof, doptr + (int64_t)qw * p.sdo.t, p.sdo.t, p.T - qw, lane);
+    float lse_q = 0.f, delta_q = 0.f;
+    if (q_pos < p.T) {
+        lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
+        delta_q = p.delta[b * p.delta_b + hd * p.delta_h + q_pos];
+    }
+    if (lse_q == -INFINITY) lse_q = 0.f;  // fully masked row: P is forced to 0 by the predicate
+
+    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
+    TileRange wr = {0, 0, 0, 0};
+    if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
+
+    f32x16 dq[DB];
+#pragma unroll
+    for (int i = 0; i < DB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dq[i][r] = 0.f;
+    const float scale = p.scale_log2;
+
+    TileStager<E, D, TK, NT> stage_k, stage_v;
+    {
+        int k0 = wg.start * TK;
+        stage_k.fetch(kptr + (int64_t)k0 * p.sk.t, p.sk.t, p.T - k0, tid);
+        stage_v.fetch(vptr + (int64_t)k0 * p.sv.t, p.sv.t, p.T - k0, tid);
+    }
+
+    for (int kt = wg.start; kt < wg.end; kt++) {
+        char* lds_k = smem + ((kt - wg.start) & 1) * 2 * TILE_BYTES;
+        char* lds_v = lds_k + TILE_BYTES;
+        stage_k.commit(lds_k, tid);
+        stage_v.commit(lds_v, tid);
+        __syncthreads();
+        if (kt + 1 < wg.end) {
+            int k1 = (kt + 1) * TK;
+            stage_k.fetch(kptr + (int64_t)k1 * p.sk.t, p.sk.t, p.T - k1, tid);
+            stage_v.fetch(vptr + (int64_t)k1 * p.sv.t, p.sv.t, p.T - k1, tid);
+        }
+        if (kt < wr.start || kt >= wr.end) continue;
+        const bool full = (kt >= wr.full_start) && (kt < wr.full_end);
+        const int k0 = kt * TK;
+
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+            f32x16 s, dp;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                s[r] = 0.f;
+                dp[r] = 0.f;
+            }
+            s = mma_rowwise<E, D>(lds_k, 32 * kb, qf, s, lane);
+            dp = mma_rowwise<E, D>(lds_v, 32 * kb, dof, dp, lane);
+            auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
+                q = q_pos;
+                k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+                lse = lse_q;
+                delta = delta_q;
+            };
+            if (full)
+                softmax_grad_block<MASK, false>(s, dp, scale, seq_len, p.margs, pos);
+            else
+                softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+                dq[db] = mma_transposed<E, D>(lds_k, 32 * kb, 32 * db, dp, dq[db], lane);
+        }
+    }
+
+    if (q_pos < p.T)
+        store_row_transposed<E, D>(dqbase + (int64_t)q_pos * p.sdq.t, dq, p.sm_scale, q_pos < seq_len, h);
+}
+
+template <typename E, int D>
+int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
+    int status = CHILL_ERR_BAD_MASK;
+    CHILL_DISPATCH_MASK(mask_id, {
+        constexpr TileConfig cfg = dq_tile_config(MASK_ID, D, Elem<E>::kDType);
+        static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+        const int n_q_tiles = cdiv(p.T, cfg.rows);
+        const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
+        if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
+        const int total = (int)total64;
+        dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
+        auto kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed>;
+        const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
+        if (cfg.lds_bytes > 48 * 1024) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)
+                return CHILL_ERR_HIP;
+        }
+        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
+        status = (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+    });
+    return status;
+}
+
+// ------------------------------------------------------------------------------------------ dK, dV
+template <typename E, int D, int MASK, int NW, int TQS>
+__global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
+                                                       int wave_has_full_blocks) {
+    using ET = typename Elem<E>::type;
+    constexpr int TKR = NW * 32;  // resident key rows per workgroup
+    constexpr int NT = NW * 64;
+    constexpr int QB = TQS / 32;
+    constexpr int DB = (D + 31) / 32;
+    constexpr int TILE_BYTES = LdsTile<E, D>::bytes(TQS);
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * TQS * 4;
+    static_assert(NT >= 2 * TQS, "LSE2 / delta staging needs one thread per value");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    if (item < 0) return;
+    const int bh = item / n_k_tiles;
+    // key tiles first-to-last: for causal-like masks the longest run first
+    const int ktile = item % n_k_tiles;
+    const int b = bh / p.H_kv;
+    const int hkv = bh % p.H_kv;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int n = lane & 31;
+    const int h = lane >> 5;
+
+    int seq_len = p.T;
+    if (p.lens != nullptr) seq_len = imin(p.lens[(int64_t)b * p.lens_stride], p.T);
+
+    const int kb0 = ktile * TKR;
+    ET* dkbase = reinterpret_cast<ET*>(p.dk) + b * p.sdk.b + hkv * p.sdk.h;
+    ET* dvbase = reinterpret_cast<ET*>(p.dv) + b * p.sdv.b + hkv * p.sdv.h;
+    if (kb0 >= seq_len) {
+        int nrows = imin(TKR, p.T - kb0);
+        zero_rows<E, D, NT>(dkbase, p.sdk.t, kb0, nrows, tid);
+        zero_rows<E, D, NT>(dvbase, p.sdv.t, kb0, nrows, tid);
+        return;
+    }
+
+    const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
+    const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
+    const int kw = kb0 + 32 * wave;
+    const int k_pos = kw + n;
+    Resident<E, D> kf, vf;
+    load_resident<E, D>(kf, kptr + (int64_t)kw * p.sk.t, p.sk.t, p.T - kw, lane);
+    load_resident<E, D>(vf, vptr + (int64_t)kw * p.sv.t, p.sv.t, p.T - kw, lane);
+
+    const TileRange wg = tile_range<MASK, false>(kb0, TKR, TQS, seq_len, false, p.margs);
+    TileRange wr = {0, 0, 0, 0};
+    if (kw < seq_len) wr = tile_range<MASK, false>(kw, 32, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
+
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int i = 0; i < DB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            dk[i][r] = 0.f;
+            dv[i][r] = 0.f;
+        }
+    const float scale = p.scale_log2;
+
+    const int n_tiles = wg.end - wg.start;
+    const int n_iters = n_tiles * p.group;
+
+    TileStager<E, D, TQS, NT> stage_q, stage_do;
+    float stage_vec = 0.f;  // thread tid < TQS stages LSE2[tid], TQS <= tid < 2*TQS stages delta
+    auto fetch = [&](int it) {
+        int g = it / n_tiles;
+        int qt = wg.start + it % n_tiles;
+        int hq = hkv * p.group + g;
+        int q0 = qt * TQS;
+        const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
+        const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
+        stage_q.fetch(qptr + (int64_t)q0 * p.sq.t, p.sq.t, p.T - q0, tid);
+        stage_do.fetch(doptr + (int64_t)q0 * p.sdo.t, p.sdo.t, p.T - q0, tid);
+        stage_vec = 0.f;
+        if (tid < 2 * TQS) {
+            int qi = q0 + (tid % TQS);
+            if (qi < p.T) {
+                if (tid < TQS) {
+                    float v = p.lse[b * p.lse_b + hq * p.lse_h + qi];
+                    stage_vec = (v == -INFINITY) ? 0.f : v;
+                } else {
+                    stage_vec = p.delta[b * p.delta_b + hq * p.delta_h + qi];
+                }
+            }
+        }
+    };
+    if (n_iters > 0) fetch(0);
+
+    for (int it = 0; it < n_iters; it++) {
+        char* lds_q = smem + (it & 1) * STAGE_BYTES;
+        char* lds_do = lds_q + TILE_BYTES;
+        float* lds_vec = reinterpret_cast<float*>(lds_do + TILE_BYTES);  // [0,TQS) LSE2, [TQS,2TQS) delta
+        stage_q.commit(lds_q, tid);
+        stage_do.commit(lds_do, tid);
+        if (tid < 2 * TQS) lds_vec[tid] = stage_vec;
+        __syncthreads();
+        if (it + 1 < n_iters) fetch(it + 1);
+        const int qt = wg.start + it % n_tiles;
+        if (qt < wr.start || qt >= wr.end) continue;
+        const bool full = (qt >= wr.full_start) && (qt < wr.full_end);
+        const int q0 = qt * TQS;
+
+#pragma unroll
+        for (int qb = 0; qb < QB; qb++) {
+            f32x16 s, dp;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                s[r] = 0.f;
+                dp[r] = 0.f;
+            }
+            s = mma_rowwise<E, D>(lds_q, 32 * qb, kf, s, lane);
+            dp = mma_rowwise<E, D>(lds_do, 32 * qb, vf, dp, lane);
+            f32x4 lse4[4], del4[4];
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                lse4[g4] = *reinterpret_cast<const f32x4*>(lds_vec + 32 * qb + 8 * g4 + 4 * h);
+                del4[g4] = *reinterpret_cast<const f32x4*>(lds_vec + TQS + 32 * qb + 8 * g4 + 4 * h);
+            }
+            auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
+                q = q0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
+                k = k_pos;
+                lse = lse4[r / 4][r % 4];
+                delta = del4[r / 4][r % 4];
+            };
+            if (full)
+                softmax_grad_block<MASK, false>(s, dp, scale, seq_len, p.margs, pos);
+            else
+                softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                dv[db] = mma_transposed<E, D>(lds_do, 32 * qb, 32 * db, s, dv[db], lane);
+                dk[db] = mma_transposed<E, D>(lds_q, 32 * qb, 32 * db, dp, dk[db], lane);
+            }
+        }
+    }
+
+    if (k_pos < p.T) {
+        const bool valid = k_pos < seq_len;
+        store_row_transposed<E, D>(dkbase + (int64_t)k_pos * p.sdk.t, dk, p.sm_scale, valid, h);
+        store_row_transposed<E, D>(dvbase + (int64_t)k_pos * p.sdv.t, dv, 1.f, valid, h);
+    }
+}
+
+template <typename E, int D>
+int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
+    int status = CHILL_ERR_BAD_MASK;
+    CHILL_DISPATCH_MASK(mask_id, {
+        constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType);
+        static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+        const int n_k_tiles = cdiv(p.T, cfg.rows);
+        const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
+        if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
+        const int total = (int)total64;
+        dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
+        auto kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed>;
+        // mask rule order is (q tile, k tile): the streamed tile is the q tile here
+        const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, 32, p.T, p.margs);
+        if (cfg.lds_bytes > 48 * 1024) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)
+                return CHILL_ERR_HIP;
+        }
+        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_k_tiles, total, hfb ? 1 : 0);
+        status = (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+    });
+    return status;
+}
+
+}  // namespace chill

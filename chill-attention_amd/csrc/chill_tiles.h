@@ -1,0 +1,55 @@
+// Static MI355X tile table: (mask id, head dim, dtype, pass) -> tile shape.  It replaces the
+// reference's per-GPU default tables and Triton autotune spaces (chill_attention/autotune.py:11-119,
+// 129-240).  The functions are constexpr so the kernel launchers instantiate exactly the shapes the
+// table reports through chill_tile_config().
+//
+// rows     = resident rows per workgroup (32 per wave): query rows in the forward and dQ passes,
+//            key rows in the dK/dV pass;
+// streamed = rows of one streamed LDS tile: keys in forward / dQ, queries in dK/dV.
+#pragma once
+
+#include "chill_params.h"
+
+namespace chill {
+
+constexpr int elem_bytes(int dtype) { return dtype == CHILL_F32 ? 4 : 2; }
+
+constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
+    (void)mask_id;
+    const bool fast16 = dtype != CHILL_F32 && D <= 128;
+    const int waves = fast16 ? 8 : 4;
+    const int streamed = fast16 ? 64 : 32;
+    // double-buffered K and V tiles
+    return TileConfig{waves * 32, streamed, waves, 2 * 2 * streamed * D * elem_bytes(dtype)};
+}
+
+constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
+    (void)mask_id;
+    const bool fast16 = dtype != CHILL_F32 && D <= 128;
+    const int waves = 4;
+    const int streamed = fast16 ? 64 : 32;
+    return TileConfig{waves * 32, streamed, waves, 2 * 2 * streamed * D * elem_bytes(dtype)};
+}
+
+constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
+    (void)mask_id;
+    const bool fast16 = dtype != CHILL_F32 && D <= 128;
+    const int waves = 4;
+    const int streamed = fast16 ? 64 : 32;
+    // double-buffered Q and dO tiles plus their LSE2 / delta vectors
+    return TileConfig{waves * 32, streamed, waves,
+                      2 * (2 * streamed * D * elem_bytes(dtype) + 2 * streamed * 4)};
+}
+
+inline int tile_config(int mask_id, int D, int dtype, int pass, TileConfig* out) {
+    if (dtype != CHILL_F32 && dtype != CHILL_F16 && dtype != CHILL_BF16) return CHILL_ERR_BAD_DTYPE;
+    if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
+    switch (pass) {
+        case CHILL_PASS_FWD: *out = fwd_tile_config(mask_id, D, dtype); return CHILL_OK;
+        case CHILL_PASS_DQ: *out = dq_tile_config(mask_id, D, dtype); return CHILL_OK;
+        case CHILL_PASS_DKDV: *out = dkdv_tile_config(mask_id, D, dtype); return CHILL_OK;
+        default: return CHILL_ERR_BAD_ARGUMENT;
+    }
+}
+
+}  // namespace chill

@@ -1,0 +1,188 @@
+/*
+ * chill_attention.h — C ABI of the MI355X (gfx950) sparse flash-attention library.
+ *
+ * This is the boundary the Python host code binds with ctypes.  Every entry point takes plain
+ * pointers, sizes and strides; no torch types cross it.  The library never allocates or frees
+ * device memory: the caller owns every buffer (outputs, the fp32 delta scratch of the backward,
+ * LSE).  All device entry points are asynchronous on the given stream and hold no mutable global
+ * state, so they are re-entrant.
+ *
+ * Each entry point cites the piece of the reference (alexdremov/chill-attention v2.1.0) whose
+ * kernel launch it replaces.
+ *
+ * Conventions
+ *   - tensors are [B, H, T, D] (q, o, do, dq) or [B, H_kv, T, D] (k, v, dk, dv); strides are in
+ *     ELEMENTS; the innermost stride must be 1 and every row start must be 16-byte aligned;
+ *   - lse / delta are fp32 [B, H, T] with element strides, innermost stride 1;
+ *   - lens is int32 [B] (element stride given) or NULL; a sequence length is min(lens[b], T);
+ *   - LSE is base-2 and includes the softmax scale: LSE2 = log2 sum_k 2^(scale*log2(e)*q.k);
+ *     a row with no unmasked key has LSE2 = -inf and O = 0;
+ *   - return value: CHILL_OK (0) or a negative ChillStatus; nothing is launched on error.
+ */
+#ifndef CHILL_ATTENTION_H
+#define CHILL_ATTENTION_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CHILL_ABI_VERSION 1
+
+typedef enum ChillStatus {
+    CHILL_OK = 0,
+    CHILL_ERR_NULL_POINTER = -1,
+    CHILL_ERR_BAD_DTYPE = -2,
+    CHILL_ERR_BAD_HEAD_DIM = -3,   /* D must be one of 16, 32, 64, 128, 256 */
+    CHILL_ERR_BAD_MASK = -4,       /* unknown mask id, wrong nargs, or argument out of range */
+    CHILL_ERR_BAD_SHAPE = -5,      /* B, H, H_kv, T non-positive or H % H_kv != 0 */
+    CHILL_ERR_BAD_STRIDE = -6,     /* inner stride != 1, negative stride, or misaligned rows */
+    CHILL_ERR_HIP = -7,            /* hipGetLastError() reported a launch failure */
+    CHILL_ERR_BAD_ARGUMENT = -8,   /* anything else (bad pass id, bad tile size, ...) */
+    CHILL_ERR_TOO_LARGE = -9       /* an index would not fit the kernels' 32-bit position math */
+} ChillStatus;
+
+typedef enum ChillDType {
+    CHILL_F32 = 0,
+    CHILL_F16 = 1,
+    CHILL_BF16 = 2
+} ChillDType;
+
+/* Mask ids: one per ChillMask class of the reference (chill_attention/mask.py:806-1394). */
+typedef enum ChillMaskId {
+    CHILL_MASK_FULL = 0,           /* FullChillMask            mask.py:806-889,   no args          */
+    CHILL_MASK_CAUSAL = 1,         /* CausalChillMask          mask.py:892-976,   no args          */
+    CHILL_MASK_SLIDING_WINDOW = 2, /* SlidingWindowChillMask   mask.py:979-1108,  (left, right)    */
+    CHILL_MASK_CHUNKWISE = 3,      /* ChunkwiseChillMask       mask.py:1111-1266, (context, back)  */
+    CHILL_MASK_PREFIX_LM = 4,      /* PrefixLMChillMask        mask.py:1269-1394, (prefix,)        */
+    CHILL_MASK_COUNT = 5
+} ChillMaskId;
+
+/* The "mask-ID-plus-args" descriptor a ChillMask instance lowers to.  The reference bakes
+ * mask.constargs into the Triton kernel as constexpr (chill.py:151); here they are runtime
+ * values, so one compiled kernel serves every instance of a mask class. */
+typedef struct ChillMaskDesc {
+    int32_t id;      /* ChillMaskId */
+    int32_t nargs;   /* number of meaningful entries of args */
+    int64_t args[4];
+} ChillMaskDesc;
+
+/* A 4-d strided tensor view (element strides). */
+typedef struct ChillTensor4 {
+    void* ptr;
+    int64_t stride[4];
+} ChillTensor4;
+
+/* Kernel passes, for chill_tile_config / chill_tile_ranges. */
+typedef enum ChillPass {
+    CHILL_PASS_FWD = 0,   /* q-tile rows, streams k-tiles   (chill_fwd.py)      */
+    CHILL_PASS_DQ = 1,    /* q-tile rows, streams k-tiles   (chill_bwd_dq.py)   */
+    CHILL_PASS_DKDV = 2   /* k-tile rows, streams q-tiles   (chill_bwd_dkdv.py) */
+} ChillPass;
+
+/* ------------------------------------------------------------------------------------------
+ * Device entry points
+ * ---------------------------------------------------------------------------------------- */
+
+/* Forward: O = softmax(mask(Q K^T * sm_scale)) V, optional LSE2.
+ * Replaces the launch of _chill_attn_fwd (chill_fwd.py:21-359) at chill.py:207, grid chill.py:122-123.
+ * `o` must be zero-initialised by the caller when lens != NULL (rows of q-tiles lying entirely
+ * at or beyond lens[b] are not written, chill_fwd.py:70-71; the adapter zero-fills at chill.py:96).
+ * `lse` may be NULL (return_lse = False). */
+int chill_fwd(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+              const ChillTensor4* o,
+              float* lse, const int64_t lse_stride[3],
+              const int32_t* lens, int64_t lens_stride,
+              int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D,
+              int32_t dtype, float sm_scale,
+              const ChillMaskDesc* mask, void* stream);
+
+/* Backward preprocessing: delta[b,h,t] = sum_d float(O[b,h,t,d]) * float(dO[b,h,t,d]).
+ * Replaces the launch of _chill_attn_bwd_precompute (utils.py:94-217) at chill.py:278-290. */
+int chill_bwd_delta(const ChillTensor4* o, const ChillTensor4* d_o,
+                    float* delta, const int64_t delta_stride[3],
+                    int32_t B, int32_t H, int32_t T, int32_t D,
+                    int32_t dtype, void* stream);
+
+/* dQ: replaces the dq branch of _chill_attn_bwd (chill_bwd.py:93-129 ->
+ * chill_bwd_dq.py:15-397), launched at chill.py:442.  `dq` is written for every row < seq_len of
+ * q-tiles that start below seq_len; the caller zero-fills it when lens != NULL (chill.py:292). */
+int chill_bwd_dq(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+                 const ChillTensor4* d_o, const ChillTensor4* dq,
+                 const float* lse, const int64_t lse_stride[3],
+                 const float* delta, const int64_t delta_stride[3],
+                 const int32_t* lens, int64_t lens_stride,
+                 int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D,
+                 int32_t dtype, float sm_scale,
+                 const ChillMaskDesc* mask, void* stream);
+
+/* dK, dV: replaces the dkdv branch of _chill_attn_bwd (chill_bwd.py:130-167 ->
+ * chill_bwd_dkdv.py:15-509), launched at chill.py:442.  One workgroup per (batch, kv head,
+ * k-tile); the GQA group loop (chill_bwd_dkdv.py:156) runs inside it.  The caller zero-fills
+ * dk / dv when lens != NULL (chill.py:293-294). */
+int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+                   const ChillTensor4* d_o, const ChillTensor4* dk, const ChillTensor4* dv,
+                   const float* lse, const int64_t lse_stride[3],
+                   const float* delta, const int64_t delta_stride[3],
+                   const int32_t* lens, int64_t lens_stride,
+                   int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D,
+                   int32_t dtype, float sm_scale,
+                   const ChillMaskDesc* mask, void* stream);
+
+/* Device-side evaluation of the mask functors, used to prove that the code the kernels run
+ * agrees bit-for-bit with the host enumeration (the role ChillMask._mask_infer, mask.py:282-330,
+ * plays for the Triton functions).  Writes `n*n` bytes (row = q, col = k) of
+ * pred(q,k) && q < n && k < n into device memory `out`. */
+int chill_mask_eval_device(const ChillMaskDesc* mask, int32_t n, uint8_t* out, void* stream);
+
+/* Device-side dump of the tile decisions of one pass for sequence length `seq_len` (<= T):
+ * for every row tile i (of `tile_in` positions) writes int32 out[i*4 + {0,1,2,3}] =
+ * {start_tile, end_tile, full_start_tile, full_end_tile} over tiles of `tile_out` positions,
+ * exactly as the kernels compute them (utils.py:221-272 and chill_fwd.py:161-185,
+ * chill_bwd_dq.py:279-293, chill_bwd_dkdv.py:329-344).  `out` is device memory,
+ * 4 * ceil(T / tile_in) int32. */
+int chill_tile_ranges_device(const ChillMaskDesc* mask, int32_t pass, int32_t T, int32_t seq_len,
+                             int32_t tile_in, int32_t tile_out, int32_t* out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Host entry points (no GPU needed)
+ * ---------------------------------------------------------------------------------------- */
+
+/* Dense mask, host memory: out[q*n + k] = pred(q,k) && q < n && k < n  (ChillMask.make_mask,
+ * mask.py:379-412). */
+int chill_mask_eval(const ChillMaskDesc* mask, int32_t n, uint8_t* out);
+
+/* Per-position inclusive limits (ChillMask._calc_limits, mask.py:414-454, without its clamp):
+ * which = 0 -> k_range_for_q(i), which = 1 -> q_range_for_k(i), for i in [0, n), evaluated with
+ * the given seq_len.  out[i*2 + {0,1}] = {lo, hi}. */
+int chill_mask_limits(const ChillMaskDesc* mask, int32_t which, int32_t n, int32_t seq_len,
+                      int32_t* out);
+
+/* Host twin of chill_tile_ranges_device (same functors compiled for the host). */
+int chill_tile_ranges(const ChillMaskDesc* mask, int32_t pass, int32_t T, int32_t seq_len,
+                      int32_t tile_in, int32_t tile_out, int32_t* out);
+
+/* is_full_block(q, k, tile_q, tile_k, seq_len) and has_full_blocks(tile_q, tile_k, seq_len) of
+ * the mask (e.g. mask.py:963-976).  Return 0/1 or a negative ChillStatus. */
+int chill_mask_is_full_block(const ChillMaskDesc* mask, int32_t q, int32_t k, int32_t tile_q,
+                             int32_t tile_k, int32_t seq_len);
+int chill_mask_has_full_blocks(const ChillMaskDesc* mask, int32_t tile_q, int32_t tile_k,
+                               int32_t seq_len);
+
+/* Static MI355X tile table, replacing autotune.py:11-119: out = {tile_rows, tile_streamed,
+ * waves_per_workgroup, lds_bytes} for (mask id, head dim, dtype, pass). */
+int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int32_t out[4]);
+
+/* Number of unmasked (q, k) pairs with q, k < T, closed form per mask — the numerator of the
+ * effective-FLOP metric (benchmark/benchmark.py:271-276 takes it from the dense mask). */
+int64_t chill_mask_nnz(const ChillMaskDesc* mask, int32_t T);
+
+const char* chill_status_string(int32_t status);
+int32_t chill_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CHILL_ATTENTION_H */
