@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X chill-attention hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--mode fwd+bwd|fwd]
+
+One "step" is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM: forward (chill_fwd) and, in fwd+bwd mode, the backward launches (chill_bwd_delta,
+chill_bwd_dkdv, chill_bwd_dq), all through the C ABI on pre-allocated buffers.  Prints ONE JSON line.
+
+  value      effective TFLOP/s over unmasked score entries (4*B*H*D*nnz forward, 2.5x for backward)
+  roofline   for the kernel that takes the largest share of the step: algorithmic FLOPs per launch
+             divided by its mean launch duration, measured here with HIP events on the launch stream
+  cpu_baseline  the reference's CPU path (dense boolean mask -> torch SDPA on the host cores), timed
+             on a bounded sample of the same workload
+
+Only one GPU is used; --gpus N with N > 1 exits with a message.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "chill-attention_amd"))
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}  # MI355X dense MFMA
+PEAK_HBM_GBS = 8000.0
+
+# name -> (mask ctor name, args, dtype, B, H, T, D, seed, sigma)
+WORKLOADS = {
+    "C1": ("CausalChillMask", (), "f32", 1, 2, 256, 64, 0, 1.0),
+    "C2": ("SlidingWindowChillMask", (128, 128), "bf16", 4, 16, 4096, 64, 1, 1.0),
+    "C3": ("CausalChillMask", (), "bf16", 8, 16, 8192, 128, 2, 1.0),
+    "C4": ("ChunkwiseChillMask", (128, 2), "f16", 2, 32, 16384, 128, 3, 0.5),
+    "C5a": ("PrefixLMChillMask", (1024,), "bf16", 4, 32, 8192, 64, 4, 1.0),
+    "C5b": ("PrefixLMChillMask", (1024,), "f32", 1, 8, 2048, 64, 4, 1.0),
+}
+
+
+def make_inputs(torch, B, H, T, D, dtype, seed, sigma, device):
+    g = torch.Generator("cpu").manual_seed(seed)
+    ts = [torch.randn(B, H, T, D, generator=g, dtype=torch.float32) * sigma for _ in range(4)]
+    return [t.to(dtype).to(device) for t in ts]  # q, k, v, dO
+
+
+class Runner:
+    """Pre-allocated buffers + raw C-ABI launches for one workload."""
+
+    def __init__(self, torch, ca, mask, q, k, v, do, sm_scale):
+        from chill_attention import _lib
+
+        self.torch, self._lib, self.mask = torch, _lib, mask
+        self.q, self.k, self.v, self.do = q, k, v, do
+        B, H, T, D = q.shape
+        self.shape = (B, H, k.shape[1], T, D)
+        self.dtype = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}[q.dtype]
+        self.o = torch.empty_like(q)
+        self.lse = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
+        self.delta = torch.empty(B, H, T, dtype=torch.float32, device=q.device)
+        self.dq, self.dk, self.dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        self.desc = mask.descriptor()
+        self.sm_scale = float(sm_scale)
+        t4 = _lib.tensor4
+        self.t = {n: t4(getattr(self, n)) for n in ("q", "k", "v", "do", "o", "dq", "dk", "dv")}
+        self.s_lse, self.s_delta = _lib.strides3(self.lse), _lib.strides3(self.delta)
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def _r(self, n):
+        return ctypes.byref(self.t[n])
+
+    def fwd(self):
+        B, H, Hkv, T, D = self.shape
+        L = self._lib
+        L.check("chill_fwd", L.lib.chill_fwd(
+            self._r("q"), self._r("k"), self._r("v"), self._r("o"), ctypes.c_void_p(self.lse.data_ptr()), self.s_lse,
+            None, 0, B, H, Hkv, T, D, self.dtype, self.sm_scale, ctypes.byref(self.desc), ctypes.c_void_p(self.stream)))
+
+    def delta_(self):
+        B, H, Hkv, T, D = self.shape
+        L = self._lib
+        L.check("chill_bwd_delta", L.lib.chill_bwd_delta(
+            self._r("o"), self._r("do"), ctypes.c_void_p(self.delta.data_ptr()), self.s_delta,
+            B, H, T, D, self.dtype, ctypes.c_void_p(self.stream)))
+
+    def dkdv(self):
+        B, H, Hkv, T, D = self.shape
+        L = self._lib
+        L.check("chill_bwd_dkdv", L.lib.chill_bwd_dkdv(
+            self._r("q"), self._r("k"), self._r("v"), self._r("do"), self._r("dk"), self._r("dv"),
+            ctypes.c_void_p(self.lse.data_ptr()), self.s_lse, ctypes.c_void_p(self.delta.data_ptr()), self.s_delta,
+            None, 0, B, H, Hkv, T, D, self.dtype, self.sm_scale, ctypes.byref(self.desc), ctypes.c_void_p(self.stream)))
+
+    def dq_(self):
+        B, H, Hkv, T, D = self.shape
+        L = self._lib
+        L.check("chill_bwd_dq", L.lib.chill_bwd_dq(
+            self._r("q"), self._r("k"), self._r("v"), self._r("do"), self._r("dq"),
+            ctypes.c_void_p(self.lse.data_ptr()), self.s_lse, ctypes.c_void_p(self.delta.data_ptr()), self.s_delta,
+            None, 0, B, H, Hkv, T, D, self.dtype, self.sm_scale, ctypes.byref(self.desc), ctypes.c_void_p(self.stream)))
+
+    def kernels(self, mode):
+        ks = [("chill_fwd", self.fwd)]
+        if mode == "fwd+bwd":
+            ks += [("chill_bwd_delta", self.delta_), ("chill_bwd_dkdv", self.dkdv), ("chill_bwd_dq", self.dq_)]
+        return ks
+
+
+def cpu_baseline(torch, mask_name, margs, dtype_name, T, D, mode, seed, sigma, budget_s=20.0):
+    """Reference CPU path on a bounded sample: dense mask -> torch SDPA (fp32 on upcast inputs, as
+    the reference's tests run it), one (batch, head) slice of the workload at full T per call."""
+    sys.path.insert(0, ROOT)
+    from oracle import chill_oracle as orc
+
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    q, k, v, do = make_inputs(torch, 1, 1, T, D, torch.float32, seed, sigma, "cpu")
+    times = []
+    t_begin = time.perf_counter()
+    while True:
+        qq, kk, vv = (x.clone().requires_grad_(mode == "fwd+bwd") for x in (q, k, v))
+        t0 = time.perf_counter()
+        out, _ = orc.reference_naive(mask_name, margs, qq, kk, vv, None)
+        if mode == "fwd+bwd":
+            out.backward(do)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_begin > budget_s or len(times) >= 4:
+            break
+    used = times[1:] if len(times) > 1 else times  # the first run warms the allocator up
+    timed = len(used)
+    sec = sum(used) / timed
+    fl = orc.flops(mask_name, margs, 1, 1, T, D, mode)
+    return {
+        "value": fl / sec / 1e12,
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"1 (batch, head) slice of the workload at full T={T}, D={D}, fp32 dense-mask torch SDPA "
+                  f"{mode}, mean of {timed} run(s), {sec:.2f} s each",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
+    ap.add_argument("--mode", default="fwd+bwd", choices=["fwd", "fwd+bwd"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures ONE MI355X; every box has one GPU and the hot path "
+                 "shards over (batch, head) without communication, so --gpus must be 1")
+
+    import torch
+
+    import chill_attention as ca
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    mask_name, margs, dname, B, H, T, D, seed, sigma = WORKLOADS[args.workload]
+    mode = "fwd" if args.workload == "C1" else args.mode
+    dtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dname]
+    mask = getattr(ca, mask_name)(*margs)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    q, k, v, do = make_inputs(torch, B, H, T, D, dtype, seed, sigma, dev)
+    run = Runner(torch, ca, mask, q, k, v, do, D ** -0.5)
+    kernels = run.kernels(mode)
+
+    for _ in range(args.warmup):
+        for _, fn in kernels:
+            fn()
+    torch.cuda.synchronize()
+
+    # per-kernel HIP events on the launch stream (torch's current stream) + whole-step wall clock
+    ev = [[(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in kernels]
+          for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        for i, (_, fn) in enumerate(kernels):
+            ev[s][i][0].record()
+            fn()
+            ev[s][i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    k_ms = [sum(ev[s][i][0].elapsed_time(ev[s][i][1]) for s in range(args.steps)) / args.steps
+            for i in range(len(kernels))]
+
+    nnz = mask.nnz(T)
+    fwd_flops = 4.0 * B * H * D * nnz
+    step_flops = fwd_flops * (3.5 if mode == "fwd+bwd" else 1.0)
+    value = step_flops / (ms_per_step * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[dname]
+
+    # algorithmic FLOPs per launch: forward 4*D per unmasked entry (2 GEMMs); of the backward's
+    # 10*D (5 GEMMs: S, dP, dV, dK, dQ) the dK/dV kernel is charged S, dP, dV, dK = 8*D and the dQ
+    # kernel dQ = 2*D (its own S and dP are recomputation, not algorithmic work)
+    per_entry = {"chill_fwd": 4.0, "chill_bwd_dkdv": 8.0, "chill_bwd_dq": 2.0, "chill_bwd_delta": 0.0}
+    es = 4 if dname == "f32" else 2
+    dom = max(range(len(kernels)), key=lambda i: k_ms[i])
+    dom_name = kernels[dom][0]
+    if dom_name == "chill_bwd_delta":
+        alg = 2.0 * B * H * T * D * es + 4.0 * B * H * T
+        roof = {"kernel": dom_name, "bound": "hbm", "achieved": alg / (k_ms[dom] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
+                "unit": "GB/s"}
+    else:
+        alg = per_entry[dom_name] * B * H * D * nnz
+        roof = {"kernel": dom_name, "bound": "mfma", "achieved": alg / (k_ms[dom] * 1e-3) / 1e12, "peak": peak,
+                "unit": "TFLOP/s"}
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = None
+    roof["avg_launch_ms"] = k_ms[dom]
+
+    out = {
+        "metric": f"effective TFLOP/s {mode}, {mask} {dname} B{B} H{H} T{T} D{D}",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dname,
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {mask} {mode} {dname} B={B} H={H} T={T} D={D} seed={seed} "
+                               f"sigma={sigma}, inputs resident in HBM"},
+        "frac_of_peak": value / peak,
+        "kernel_ms": {kernels[i][0]: k_ms[i] for i in range(len(kernels))},
+        "fwd_tflops": fwd_flops / (k_ms[0] * 1e-3) / 1e12,
+        "fwd_frac_of_peak": fwd_flops / (k_ms[0] * 1e-3) / 1e12 / peak,
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, mask_name, margs, dname, T, D, mode, seed, sigma)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
