@@ -341,7 +341,7 @@ def reference_naive(name, args, q, k, v, lens=None):
         v = v.repeat_interleave(g, dim=1)
     B, _, T, _ = q.shape
     lens_np = None if lens is None else lens.detach().cpu().numpy()
-    attn_mask = torch.from_numpy(np.ascontiguousarray(_full_mask(name, args, B, T, lens_np))).to(q.device)
+    attn_mask = torch.from_numpy(np.array(_full_mask(name, args, B, T, lens_np))).to(q.device)
     if lens is None:
         res_mask = torch.as_tensor(1, device=q.device)
     else:

@@ -1,0 +1,131 @@
+"""The C-ABI shared library on the CPU: it loads, exports every symbol the header declares, and its
+argument validation answers with error codes before anything is launched (no GPU needed)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from chill_attention import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "chill_attention.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(chill_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 15
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"{n} declared in include/chill_attention.h but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names
+    assert _lib.lib.chill_abi_version() == _lib.ABI_VERSION
+
+
+def test_status_strings():
+    for code in range(0, -10, -1):
+        s = _lib.lib.chill_status_string(code).decode()
+        assert s and s != "unknown status"
+    assert _lib.lib.chill_status_string(-99).decode() == "unknown status"
+
+
+def _t4(ptr=0x1000, strides=(1 << 20, 1 << 16, 128, 1)):
+    t = _lib.ChillTensor4()
+    t.ptr = ptr
+    for i, s in enumerate(strides):
+        t.stride[i] = s
+    return t
+
+
+def _call_fwd(q=None, k=None, v=None, o=None, B=1, H=2, Hkv=2, T=64, D=128, dtype=_lib.BF16, mask=None, null_q=False):
+    q, k, v, o = (x if x is not None else _t4() for x in (q, k, v, o))
+    mask = mask if mask is not None else _lib.mask_desc(_lib.MASK_CAUSAL, [])
+    s3 = (ctypes.c_int64 * 3)(H * T, T, 1)
+    return _lib.lib.chill_fwd(
+        None if null_q else ctypes.byref(q), ctypes.byref(k), ctypes.byref(v), ctypes.byref(o), None, s3, None, 0,
+        B, H, Hkv, T, D, dtype, 0.1, ctypes.byref(mask), None)
+
+
+def test_forward_validation_returns_codes_without_launching():
+    E = {"null": -1, "dtype": -2, "dim": -3, "mask": -4, "shape": -5, "stride": -6, "large": -9}
+    assert _call_fwd(null_q=True) == E["null"]
+    assert _call_fwd(q=_t4(ptr=None)) == E["null"]
+    assert _call_fwd(dtype=7) == E["dtype"]
+    assert _call_fwd(D=48) == E["dim"]
+    assert _call_fwd(D=0) == E["dim"]
+    assert _call_fwd(mask=_lib.mask_desc(9, [])) == E["mask"]
+    assert _call_fwd(mask=_lib.mask_desc(_lib.MASK_SLIDING_WINDOW, [3])) == E["mask"]  # wrong arg count
+    assert _call_fwd(mask=_lib.mask_desc(_lib.MASK_CHUNKWISE, [0, 1])) == E["mask"]  # zero chunk size
+    assert _call_fwd(mask=_lib.mask_desc(_lib.MASK_PREFIX_LM, [-1])) == E["mask"]
+    assert _call_fwd(B=0) == E["shape"]
+    assert _call_fwd(H=6, Hkv=4) == E["shape"]
+    assert _call_fwd(T=(1 << 29) + 1) == E["large"]
+    assert _call_fwd(q=_t4(strides=(1 << 20, 1 << 16, 128, 2))) == E["stride"]  # inner stride
+    assert _call_fwd(q=_t4(strides=(1 << 20, 1 << 16, 100, 1))) == E["stride"]  # rows not 16-byte aligned
+    assert _call_fwd(q=_t4(ptr=0x1004)) == E["stride"]  # misaligned base
+    assert _call_fwd(q=_t4(strides=(-1, 1 << 16, 128, 1))) == E["stride"]
+    with pytest.raises(_lib.ChillLibraryError) as ei:
+        _lib.check("chill_fwd", _call_fwd(D=48))
+    assert ei.value.status == E["dim"] and "head dim" in str(ei.value)
+
+
+def test_backward_and_debug_validation():
+    t = _t4()
+    s3 = (ctypes.c_int64 * 3)(128, 64, 1)
+    m = _lib.mask_desc(_lib.MASK_CAUSAL, [])
+    assert _lib.lib.chill_bwd_delta(ctypes.byref(t), ctypes.byref(t), None, s3, 1, 2, 64, 128, _lib.BF16, None) == -1
+    assert _lib.lib.chill_bwd_delta(ctypes.byref(t), ctypes.byref(t), 0x1000, s3, 1, 2, 64, 100, _lib.BF16, None) == -3
+    bad_s3 = (ctypes.c_int64 * 3)(128, 64, 2)
+    assert _lib.lib.chill_bwd_delta(ctypes.byref(t), ctypes.byref(t), 0x1000, bad_s3, 1, 2, 64, 128, _lib.BF16, None) == -6
+    r = _lib.lib.chill_bwd_dq(ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), ctypes.byref(t),
+                              None, s3, 0x1000, s3, None, 0, 1, 2, 2, 64, 128, _lib.BF16, 0.1, ctypes.byref(m), None)
+    assert r == -1  # lse missing
+    r = _lib.lib.chill_bwd_dkdv(ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), None,
+                                0x1000, s3, 0x1000, s3, None, 0, 1, 2, 2, 64, 128, _lib.BF16, 0.1, ctypes.byref(m), None)
+    assert r == -1  # dv missing
+    assert _lib.lib.chill_mask_eval_device(ctypes.byref(m), 16, None, None) == -1
+    assert _lib.lib.chill_tile_ranges_device(ctypes.byref(m), 5, 64, 64, 32, 32, 0x1000, None) == -8
+    out = (ctypes.c_int32 * 8)()
+    assert _lib.lib.chill_tile_ranges(ctypes.byref(m), 0, 64, 65, 32, 32, out) == -5  # seq_len > T
+    assert _lib.lib.chill_tile_ranges(ctypes.byref(m), 0, 64, 64, 0, 32, out) == -8
+    assert _lib.lib.chill_mask_limits(ctypes.byref(m), 2, 4, 4, out) == -8
+
+
+def test_tile_table():
+    import torch
+
+    import chill_attention as ca
+    from chill_attention.tiles import _get_default_config_bwd, _get_default_config_fwd, tile_config
+
+    for mask in (ca.CausalChillMask(), ca.SlidingWindowChillMask(1, 1)):
+        for dt in (torch.float32, torch.float16, torch.bfloat16):
+            for D in (16, 32, 64, 128, 256):
+                for p in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKDV):
+                    c = tile_config(mask, D, dt, p)
+                    assert c["rows"] == 32 * c["waves"] and c["streamed"] % 32 == 0
+                    assert 0 < c["lds_bytes"] <= 160 * 1024
+    tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
+    assert tq == 32 * waves
+    (dq_q, dq_k, _), (dk_q, dk_k, _) = _get_default_config_bwd(128, torch.bfloat16)
+    assert dq_q % 32 == 0 and dk_k % 32 == 0
+    out = (ctypes.c_int32 * 4)()
+    assert _lib.lib.chill_tile_config(0, 100, _lib.BF16, 0, out) == -3
+    assert _lib.lib.chill_tile_config(0, 64, 5, 0, out) == -2
+    assert _lib.lib.chill_tile_config(9, 64, _lib.BF16, 0, out) == -4
+    assert _lib.lib.chill_tile_config(0, 64, _lib.BF16, 3, out) == -8
+
+
+def test_cpu_tensors_are_refused():
+    import torch
+
+    import chill_attention as ca
+
+    q = torch.randn(1, 1, 16, 16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        ca.chill_attention(q, q, q, mask=ca.CausalChillMask())

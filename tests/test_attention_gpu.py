@@ -1,0 +1,237 @@
+"""GPU parity tests: the HIP path (through the public op, i.e. through the C ABI) against the oracle.
+
+The matrix mirrors the reference's test_simple_chill_forward / test_simple_chill_backward
+(test/test_chill_attention.py:84-329): five masks x three dtypes x lens {none, tricky, random} x
+contiguous / non-contiguous inputs x head dims x batch sizes x GQA shapes x sequence lengths, with
+the reference's own tolerances.  The oracle (dense mask -> torch SDPA on fp32-upcast inputs, autograd
+for the gradients) runs on the same device tensors.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import chill_attention as ca
+from conftest import MASK_INSTANCES, make_mask, mask_id
+from oracle import chill_oracle as orc
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+# reference tolerances (atol, rtol): test_chill_attention.py:167-172 (outputs), :316-321 (gradients)
+OUT_TOL = {torch.float32: (2e-6, 1e-4), torch.float16: (1e-2, 1e-3), torch.bfloat16: (5e-2, 1e-2)}
+GRAD_TOL = {torch.float32: (5e-5, 1e-3), torch.float16: (5e-3, 1e-3), torch.bfloat16: (1e-1, 1e-2)}
+
+
+def make_lens(kind, B, T, rng):
+    """test_chill_attention.py:38-58"""
+    if kind == "none":
+        return None
+    if kind == "tricky":
+        choices = [1, 2, 5, T + 1, T, max(T // 2, 1), max(T // 4, 1)]
+        vals = rng.choice(choices, B)
+    else:
+        vals = rng.integers(1, T + 1, B)
+    return torch.tensor(vals, dtype=torch.int32, device=DEV)
+
+
+def make_qkv(shape, dtype, noncontiguous):
+    t = torch.testing.make_tensor(shape, dtype=dtype, device=DEV, noncontiguous=noncontiguous, low=-0.1, high=0.1)
+    t.normal_()
+    return t
+
+
+# (noncontiguous, head_dim, B, (H, H_kv)) combinations covering every value of the reference matrix
+FWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (6, 3)), (False, 128, 1, (6, 1)), (True, 16, 7, (8, 8))]
+BWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (8, 2)), (False, 128, 16, (6, 1)), (True, 16, 7, (8, 8)),
+              (False, 128, 1, (8, 1))]
+
+
+@pytest.mark.parametrize("T", [1, 10, 16, 500, 512], ids=lambda x: f"time-{x}")
+@pytest.mark.parametrize("lens_kind", ["none", "tricky", "random"], ids=lambda x: f"lens-{x}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("m", MASK_INSTANCES[:5], ids=mask_id)
+def test_forward_matrix(m, dtype, lens_kind, T):
+    mask = make_mask(m)
+    rng = np.random.default_rng(hash((m[0], str(dtype), lens_kind, T)) % (1 << 32))
+    for noncontig, D, B, (H, Hkv) in FWD_SHAPES:
+        print(f"fwd {mask} {dtype} lens={lens_kind} T={T} noncontig={noncontig} D={D} B={B} H={H}/{Hkv}", flush=True)
+        q = make_qkv((B, H, T, D), dtype, noncontig)
+        k = make_qkv((B, Hkv, T, D), dtype, noncontig)
+        v = make_qkv((B, Hkv, T, D), dtype, noncontig)
+        lens = make_lens(lens_kind, B, T, rng)
+        ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), lens)
+        out = ca.chill_attention(q, k, v, mask=mask, lens=lens) * res_mask
+        atol, rtol = OUT_TOL[dtype]
+        torch.testing.assert_close(out, ref.to(dtype), atol=atol, rtol=rtol)
+
+
+@pytest.mark.parametrize("T", [1, 10, 16, 800, 1025], ids=lambda x: f"time-{x}")
+@pytest.mark.parametrize("lens_kind", ["none", "tricky", "random"], ids=lambda x: f"lens-{x}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("m", MASK_INSTANCES[:5], ids=mask_id)
+def test_backward_matrix(m, dtype, lens_kind, T):
+    mask = make_mask(m)
+    rng = np.random.default_rng(hash((m[0], str(dtype), lens_kind, T, "b")) % (1 << 32))
+    for noncontig, D, B, (H, Hkv) in BWD_SHAPES:
+        if T >= 800 and B == 16:
+            B = 3  # keeps the dense oracle of the longest cases small; B=16 is covered at short T
+        print(f"bwd {mask} {dtype} lens={lens_kind} T={T} noncontig={noncontig} D={D} B={B} H={H}/{Hkv}", flush=True)
+        q = make_qkv((B, H, T, D), dtype, noncontig).requires_grad_()
+        k = make_qkv((B, Hkv, T, D), dtype, noncontig).requires_grad_()
+        v = make_qkv((B, Hkv, T, D), dtype, noncontig).requires_grad_()
+        lens = make_lens(lens_kind, B, T, rng)
+        qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+        ref, res_mask = orc.reference_naive(m[0], m[1], qf, kf, vf, lens)
+        dout = make_qkv((B, H, T, D), torch.float32, noncontig)
+        dout = dout * res_mask.broadcast_to(dout.shape)
+        ref.backward(dout)
+        out = ca.chill_attention(q, k, v, mask=mask, lens=lens)
+        out.backward(dout.to(dtype) if dtype != torch.float32 else dout)
+        atol, rtol = OUT_TOL[dtype]
+        torch.testing.assert_close(out.detach() * res_mask, ref.detach().to(dtype), atol=atol, rtol=rtol)
+        atol, rtol = GRAD_TOL[dtype]
+        for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
+            assert torch.isfinite(got).all(), name
+            torch.testing.assert_close(got, want.to(dtype), atol=atol, rtol=rtol, msg=lambda s: f"{name}: {s}")
+
+
+@pytest.mark.parametrize("D", [32, 64, 256])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+def test_other_head_dims(dtype, D):
+    for m in (MASK_INSTANCES[1], MASK_INSTANCES[3]):
+        mask = make_mask(m)
+        B, H, Hkv, T = 2, 4, 2, 333
+        q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
+        qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+        ref, _ = orc.reference_naive(m[0], m[1], qf, kf, vf, None)
+        dout = torch.randn_like(ref)
+        ref.backward(dout)
+        out = ca.chill_attention(q, k, v, mask=mask)
+        out.backward(dout.to(dtype))
+        torch.testing.assert_close(out.detach(), ref.detach().to(dtype), atol=OUT_TOL[dtype][0], rtol=OUT_TOL[dtype][1])
+        for got, want in ((v.grad, vf.grad), (k.grad, kf.grad), (q.grad, qf.grad)):
+            torch.testing.assert_close(got, want.to(dtype), atol=GRAD_TOL[dtype][0], rtol=GRAD_TOL[dtype][1])
+
+
+def test_lse_and_fully_masked_rows():
+    """LSE2 is base 2 and includes the scale (chill_fwd.py:328); rows that see no key give O = 0 and
+    LSE2 = -inf; rows at or beyond lens give O = 0."""
+    m = ("SlidingWindowChillMask", (3, 0))
+    mask = make_mask(m)
+    B, H, T, D = 2, 2, 200, 64
+    q, k, v = (torch.randn(B, H, T, D, device=DEV) for _ in range(3))
+    lens = torch.tensor([200, 37], dtype=torch.int32, device=DEV)
+    o, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens, sm_scale=0.2, return_lse=True)
+    ref = orc.attention_f64(m[0], m[1], q.cpu().numpy(), k.cpu().numpy(), v.cpu().numpy(), lens=lens.cpu().numpy(), sm_scale=0.2)
+    assert lse.shape == (B, H, T) and lse.dtype == torch.float32
+    np.testing.assert_allclose(lse[0].cpu().numpy(), ref["lse2"][0], atol=2e-5, rtol=1e-5)
+    np.testing.assert_allclose(lse[1, :, :37].cpu().numpy(), ref["lse2"][1, :, :37], atol=2e-5, rtol=1e-5)
+    np.testing.assert_allclose(o.cpu().numpy(), ref["o"], atol=2e-5, rtol=1e-4)
+    assert (o[1, :, 37:] == 0).all()
+    # a mask under which late rows see nothing once lens cuts the keys: chunk 0 only is valid
+    m2 = ("ChunkwiseChillMask", (16, 0))
+    lens2 = torch.tensor([16, 200], dtype=torch.int32, device=DEV)
+    o2, lse2 = ca.chill_attention(q, k, v, mask=make_mask(m2), lens=lens2, return_lse=True)
+    assert (o2[0, :, 16:] == 0).all() and torch.isfinite(o2).all()
+    # sm_scale default and custom agree with the closed form
+    o3 = ca.chill_attention(q, k, v, mask=ca.FullChillMask(), sm_scale=D ** -0.5)
+    o4 = ca.chill_attention(q, k, v, mask=ca.FullChillMask())
+    assert torch.equal(o3, o4)
+
+
+def test_rows_without_keys():
+    """A query whose keys are all masked (possible with lens cutting a window that only looks ahead)."""
+    m = ("SlidingWindowChillMask", (0, 0))
+    B, H, T, D = 1, 1, 64, 32
+    q, k, v = (torch.randn(B, H, T, D, device=DEV) for _ in range(3))
+    o, lse = ca.chill_attention(q, k, v, mask=make_mask(m), return_lse=True)
+    torch.testing.assert_close(o, v, atol=1e-6, rtol=1e-6)  # each row sees only itself
+    expected = (q * k).sum(-1) * D ** -0.5 * math.log2(math.e)
+    torch.testing.assert_close(lse, expected, atol=1e-4, rtol=1e-5)
+
+
+def test_strided_views_run_without_copy_and_match():
+    """[B, T, H, D] storage viewed as [B, H, T, D] (unit inner stride) is consumed in place."""
+    mask = ca.CausalChillMask()
+    B, H, T, D = 2, 4, 300, 64
+    base = [torch.randn(B, T, H, D, device=DEV, dtype=torch.bfloat16) for _ in range(3)]
+    q, k, v = (x.transpose(1, 2) for x in base)
+    assert not q.is_contiguous()
+    out = ca.chill_attention(q, k, v, mask=mask)
+    out_c = ca.chill_attention(q.contiguous(), k.contiguous(), v.contiguous(), mask=mask)
+    assert torch.equal(out, out_c)
+    # slices with a storage offset and a padded row pitch
+    big = torch.randn(B, H, T, 2 * D, device=DEV, dtype=torch.bfloat16)
+    qs, ks, vs = big[..., :D], big[..., D:], big[..., :D]
+    out_s = ca.chill_attention(qs, ks, vs, mask=mask)
+    assert torch.equal(out_s, ca.chill_attention(qs.contiguous(), ks.contiguous(), vs.contiguous(), mask=mask))
+
+
+def test_gradients_through_strided_and_fp32_dout():
+    mask = ca.PrefixLMChillMask(20)
+    B, H, T, D = 2, 2, 130, 32
+    q, k, v = (torch.randn(B, T, H, D, device=DEV, dtype=torch.float16).transpose(1, 2).requires_grad_() for _ in range(3))
+    out = ca.chill_attention(q, k, v, mask=mask)
+    dout = torch.randn(B, H, T, D, device=DEV, dtype=torch.float32)
+    out.backward(dout)  # fp32 upstream gradient, as the reference's test passes it
+    qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+    ref, _ = orc.reference_naive("PrefixLMChillMask", (20,), qf, kf, vf, None)
+    ref.backward(dout)
+    for got, want in ((q.grad, qf.grad), (k.grad, kf.grad), (v.grad, vf.grad)):
+        torch.testing.assert_close(got, want.half(), atol=5e-3, rtol=1e-3)
+
+
+def test_mask_args_are_runtime_values():
+    """Instances of one mask class share one registered op; their arguments reach the kernel at run time."""
+    q, k, v = (torch.randn(1, 2, 256, 64, device=DEV, dtype=torch.float16) for _ in range(3))
+    a = ca.chill_attention(q, k, v, mask=ca.SlidingWindowChillMask(5, 1))
+    b = ca.chill_attention(q, k, v, mask=ca.SlidingWindowChillMask(50, 20))
+    ra, _ = orc.reference_naive("SlidingWindowChillMask", (5, 1), q.float(), k.float(), v.float())
+    rb, _ = orc.reference_naive("SlidingWindowChillMask", (50, 20), q.float(), k.float(), v.float())
+    torch.testing.assert_close(a, ra.half(), atol=1e-2, rtol=1e-3)
+    torch.testing.assert_close(b, rb.half(), atol=1e-2, rtol=1e-3)
+    assert hasattr(torch.ops.chill_attention, "forwardSlidingWindowChillMask")
+    assert hasattr(torch.ops.chill_attention, "backwardSlidingWindowChillMask")
+
+
+def test_opcheck_and_compile():
+    mask = ca.CausalChillMask()
+    ca.register_chill_mask(mask)
+    q, k, v = (torch.randn(1, 2, 64, 32, device=DEV, dtype=torch.float32, requires_grad=True) for _ in range(3))
+    torch.library.opcheck(
+        torch.ops.chill_attention.forwardCausalChillMask.default,
+        (q, k, v, None, [], 0.17, True, False, "ieee", False),
+        test_utils=("test_schema", "test_faketensor", "test_autograd_registration"),
+    )
+    fn = torch.compile(lambda a, b, c: ca.chill_attention(a, b, c, mask=mask), fullgraph=True)
+    out = fn(q, k, v)
+    torch.testing.assert_close(out, ca.chill_attention(q, k, v, mask=mask))
+    out.sum().backward()
+    assert q.grad is not None and torch.isfinite(q.grad).all()
+
+
+def test_device_functors_equal_host():
+    """The mask functors and tile decisions as executed ON THE GPU equal the host build bit for bit."""
+    import ctypes
+
+    from chill_attention import _lib
+
+    for m in MASK_INSTANCES:
+        mask = make_mask(m)
+        desc = mask.descriptor()
+        for n in (1, 33, 500, 1030):
+            out = torch.empty(n, n, dtype=torch.uint8, device=DEV)
+            _lib.check("chill_mask_eval_device", _lib.lib.chill_mask_eval_device(
+                ctypes.byref(desc), n, ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+            assert torch.equal(out.bool().cpu(), mask.make_mask(n).cpu())
+        for pass_id in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKDV):
+            for T, seq_len, tin, tout in ((1030, 1030, 32, 64), (1030, 517, 256, 64), (8192, 8192, 128, 64), (300, 1, 32, 32)):
+                n_tiles = -(-T // tin)
+                out = torch.empty(n_tiles, 4, dtype=torch.int32, device=DEV)
+                _lib.check("chill_tile_ranges_device", _lib.lib.chill_tile_ranges_device(
+                    ctypes.byref(desc), pass_id, T, seq_len, tin, tout, ctypes.c_void_p(out.data_ptr()),
+                    ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+                assert torch.equal(out.cpu(), mask._calc_tile_ranges(T, tin, tout, pass_id, seq_len))
