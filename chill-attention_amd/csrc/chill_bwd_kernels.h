@@ -139,6 +139,8 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
 
     const int qw = qb + 32 * wave;
     const int q_pos = qw + n;
+    OperandOffsets<E, D> ofs;
+    ofs.init(lane);
     Resident<E, D> qf, dof;
     load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
     load_resident<E, D>(dof, doptr + (int64_t)qw * p.sdo.t, p.sdo.t, p.T - qw, lane);
@@ -190,8 +192,8 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
                 s[r] = 0.f;
                 dp[r] = 0.f;
             }
-            s = mma_rowwise<E, D>(lds_k, 32 * kb, qf, s, lane);
-            dp = mma_rowwise<E, D>(lds_v, 32 * kb, dof, dp, lane);
+            s = mma_rowwise<E, D>(lds_k, kb, ofs, qf, s, lane);
+            dp = mma_rowwise<E, D>(lds_v, kb, ofs, dof, dp, lane);
             auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
                 q = q_pos;
                 k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
                 softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
 #pragma unroll
             for (int db = 0; db < DB; db++)
-                dq[db] = mma_transposed<E, D>(lds_k, 32 * kb, 32 * db, dp, dq[db], lane);
+                dq[db] = mma_transposed<E, D>(lds_k, kb, db, ofs, dp, dq[db], lane);
         }
     }
 
@@ -281,6 +283,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
     const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
     const int kw = kb0 + 32 * wave;
     const int k_pos = kw + n;
+    OperandOffsets<E, D> ofs;
+    ofs.init(lane);
     Resident<E, D> kf, vf;
     load_resident<E, D>(kf, kptr + (int64_t)kw * p.sk.t, p.sk.t, p.T - kw, lane);
     load_resident<E, D>(vf, vptr + (int64_t)kw * p.sv.t, p.sv.t, p.T - kw, lane);
@@ -350,8 +354,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
                 s[r] = 0.f;
                 dp[r] = 0.f;
             }
-            s = mma_rowwise<E, D>(lds_q, 32 * qb, kf, s, lane);
-            dp = mma_rowwise<E, D>(lds_do, 32 * qb, vf, dp, lane);
+            s = mma_rowwise<E, D>(lds_q, qb, ofs, kf, s, lane);
+            dp = mma_rowwise<E, D>(lds_do, qb, ofs, vf, dp, lane);
             f32x4 lse4[4], del4[4];
 #pragma unroll
             for (int g4 = 0; g4 < 4; g4++) {
@@ -370,8 +374,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
                 softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
 #pragma unroll
             for (int db = 0; db < DB; db++) {
-                dv[db] = mma_transposed<E, D>(lds_do, 32 * qb, 32 * db, s, dv[db], lane);
-                dk[db] = mma_transposed<E, D>(lds_q, 32 * qb, 32 * db, dp, dk[db], lane);
+                dv[db] = mma_transposed<E, D>(lds_do, qb, db, ofs, s, dv[db], lane);
+                dk[db] = mma_transposed<E, D>(lds_q, qb, db, ofs, dp, dk[db], lane);
             }
         }
     }

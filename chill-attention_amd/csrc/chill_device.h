@@ -35,6 +35,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 
 typedef __attribute__((address_space(3))) i16x4 lds_i16x4;
+typedef __attribute__((address_space(3))) i32x4 lds_i32x4;
+typedef __attribute__((address_space(3))) char lds_char;
+typedef __attribute__((address_space(3))) float lds_float;
 
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -125,16 +128,25 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 // ------------------------------------------------------------------------------------------
 // LDS tile: ROWS x D elements, addressed in 16-byte chunks.  Chunk (row, c) has linear index
-// L = row * CH + c and lives at phys(L) = L with its low four bits XORed by the next four, a
-// bijection inside every aligned group of 16 chunks (256 bytes).  Lanes that read the same chunk
-// column of consecutive rows (the row-wise A operand) land in different banks.
+// L = row * CH + c and lives at phys(L) = L ^ g(key), where key is the index of the 256-byte line
+// (of the row, for rows longer than a line) and g swaps the two 2-bit halves of key & 15.  The XOR
+// only touches the low four bits of L, so it is an involution inside every aligned group of 16
+// chunks.  Measured on gfx950 (64 banks x 4 B; a 16-byte read serves 16 lanes per cycle, an 8-byte
+// read 32 lanes per cycle) both access patterns of the kernels are conflict-free with it:
+//   * row-wise operand: 16 consecutive rows, same chunk column -> g(key) takes 16 values;
+//   * transposed operand: 4 consecutive rows x 64 contiguous bytes -> bits 2..3 of g(key), the
+//     64-byte segment index, take 4 values.
 // ------------------------------------------------------------------------------------------
 template <typename E, int D>
 struct LdsTile {
     static constexpr int CH = D * Elem<E>::kBytes / 16;  // chunks per row
-    static_assert(CH >= 1, "row shorter than one chunk");
+    static_assert(CH >= 2, "row shorter than two chunks");
+    static constexpr int BLOCK_BYTES = 32 * CH * 16;     // 32 rows
+    // +32 rows leaves the swizzle key unchanged (mod 16) when 32 rows are a multiple of 16 lines
+    static constexpr bool kBlockAffine = CH >= 8;
 
-    __device__ __forceinline__ static int phys(int L) { return L ^ ((L >> 4) & 15); }
+    __device__ __forceinline__ static int swz(int t) { return ((t & 3) << 2) | ((t >> 2) & 3); }
+    __device__ __forceinline__ static int phys(int L) { return L ^ swz(CH > 16 ? (L >> 5) : (L >> 4)); }
     __device__ __forceinline__ static int chunk_off(int row, int c) { return phys(row * CH + c) * 16; }
     // byte offset of element (row, col)
     __device__ __forceinline__ static int elem_off(int row, int col) {
@@ -183,69 +195,133 @@ struct TileStager {
     }
 };
 
-// Row-wise A/B operand: the 16-byte chunk (row, 2*j + h).  For 16-bit types that is one MFMA
-// operand (contraction slots 16*j + 8*h ..), for fp32 four of them (slots 8*j + 4*h ..).
-template <typename E, int D>
-__device__ __forceinline__ i32x4 lds_row_chunk(const char* lds, int row, int c) {
-    return *reinterpret_cast<const i32x4*>(lds + LdsTile<E, D>::chunk_off(row, c));
-}
-
-// Transposed A operand for 16-bit types, built from two ds_read_b64_tr_b16.
-// That instruction works on groups of 16 lanes: lane r of a group supplies the address of four
-// consecutive 16-bit elements X[k0 + r/4][n0 + 4*(r%4) ..], and lane i of the group receives
-// X[k0 + 0..3][n0 + i].  Here: rows = contraction index (4 consecutive rows per read), the wave's
-// 32 output rows n split into two groups of 16 columns.
-// Returns the operand for rows {row0 + 4*h + (0..3), row0 + 8 + 4*h + (0..3)} at column col0 + n.
-template <typename E, int D>
-__device__ __forceinline__ i32x4 lds_tr_operand(const char* lds, int row0, int col0, int lane) {
+// Asynchronous staging of a ROWS x D tile straight into LDS (global_load_lds_dwordx4): no
+// registers, no ds_write.  One wave instruction fills a 1 KiB slab: lane l's 16 bytes land at
+// slab base + 16*l, so the lane FETCHES the logical chunk whose swizzled position is its slot.
+// Rows >= rows_valid are zero-filled with ordinary LDS stores.  The caller waits with
+// wait_async_tiles() and then a workgroup barrier before anyone reads the tile.
+template <typename E, int D, int ROWS, int NT>
+struct AsyncTile {
     typedef LdsTile<E, D> L;
-    int h = lane >> 5;
-    int r = lane & 15;
-    int colgrp = (lane >> 4) & 1;
-    int col = col0 + 16 * colgrp + 4 * (r & 3);
-    if (D < 32) col &= (D - 1);
-    int row = row0 + 4 * h + (r >> 2);
-    const lds_i16x4* p0 = (const lds_i16x4*)(lds + L::elem_off(row, col));
-    const lds_i16x4* p1 = (const lds_i16x4*)(lds + L::elem_off(row + 8, col));
-    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)p0);
-    i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)p1);
-    i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(i32x4, v);
-}
+    static constexpr int TOTAL = ROWS * L::CH;  // chunks, a multiple of 64
+    static constexpr int SLABS = TOTAL / 64;
+    static constexpr int NWV = NT / 64;
+    static constexpr int PER_WAVE = (SLABS + NWV - 1) / NWV;
+    static_assert(TOTAL % 64 == 0, "tile must be a whole number of 1 KiB slabs");
 
-// acc(32 out-rows x 32 cols) += X^T(rows of the LDS tile [row0, row0+32) as contraction) * P,
-// where P is a 32x32 accumulator-layout block (rows = contraction index) reused as B operand.
-// Output row index = column of the LDS tile (col0 + n).
-template <typename E, int D>
-__device__ __forceinline__ f32x16 mma_transposed(const char* lds, int row0, int col0, f32x16 p,
-                                                 f32x16 acc, int lane) {
-    if constexpr (Elem<E>::k16) {
+    __device__ __forceinline__ static void issue(const typename Elem<E>::type* base, int64_t row_stride,
+                                                 int rows_valid, char* lds, int wave, int lane) {
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            f32x8 ps;
-#pragma unroll
-            for (int e = 0; e < 8; e++) ps[e] = p[8 * s + e];
-            i32x4 b = Elem<E>::pack8(ps);
-            i32x4 a = lds_tr_operand<E, D>(lds, row0 + 16 * s, col0, lane);
-            acc = Elem<E>::mma(a, b, acc);
-        }
-    } else {
-        typedef LdsTile<E, D> L;
-        int h = lane >> 5;
-        int col = col0 + (lane & 31);
-        if (D < 32) col &= (D - 1);
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            int row = row0 + 8 * (r / 4) + 4 * h + (r % 4);
-            float a = *reinterpret_cast<const float*>(lds + L::elem_off(row, col));
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, p[r], acc, 0, 0, 0);
+        for (int i = 0; i < PER_WAVE; i++) {
+            int slab = i * NWV + wave;
+            if (SLABS % NWV == 0 || slab < SLABS) {
+                int slot = slab * 64 + lane;
+                int lg = L::phys(slot);  // the swizzle is an involution
+                int row = lg / L::CH;
+                int c = lg % L::CH;
+                if (row < rows_valid) {
+                    const char* g = reinterpret_cast<const char*>(base + (int64_t)row * row_stride) + c * 16;
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void*)g,
+                        (__attribute__((address_space(3))) void*)(lds + slab * 1024), 16, 0, 0);
+                } else {
+                    *reinterpret_cast<i32x4*>(lds + slot * 16) = i32x4{0, 0, 0, 0};
+                }
+            }
         }
     }
-    return acc;
+};
+
+// All asynchronous tile loads issued so far by this wave have landed in LDS.
+__device__ __forceinline__ void wait_async_tiles() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// ------------------------------------------------------------------------------------------
+// Padded LDS tile: rows of D elements at a pitch of RB + PAD bytes.  Addresses are affine in
+// (row, column), so every LDS read of the inner loops is "per-lane base register + immediate".
+// Used where a tile is read in one pattern only (forward: K row-wise, V transposed); the pad is
+// chosen per pattern (measured on gfx950, 64 banks x 4 B):
+//   * row-wise 16-byte reads (16 lanes = 16 consecutive rows per cycle): PAD = 16;
+//   * transposed 8-byte reads (32 lanes = 4 consecutive rows x 64 bytes per cycle): pitch = 64 mod 256;
+//   * fp32 column reads (two rows four apart per cycle): pitch = 32 mod 64.
+// ------------------------------------------------------------------------------------------
+template <typename E, int D, int PAD>
+struct PaddedTile {
+    static constexpr int RB = D * Elem<E>::kBytes;
+    static constexpr int CH = RB / 16;
+    static constexpr int PITCH = RB + PAD;
+    static constexpr int CHP = PITCH / 16;  // 16-byte slots per row, padding included
+    static_assert(PAD % 16 == 0, "pad in whole chunks");
+    static constexpr int bytes(int rows) { return rows * PITCH; }
+};
+
+template <typename E, int D>
+constexpr int rowwise_pad() { return 16; }
+template <typename E, int D>
+constexpr int transposed_pad() {
+    return Elem<E>::k16 ? (D * Elem<E>::kBytes >= 128 ? 64 : 0) : 32;
 }
 
-// acc(32 rows of the LDS tile x 32 cols) += X[row0 + 0..31][:] * B^T where the B operand chunks
-// (resident rows, e.g. the wave's Q rows) live in registers: b.c[j] = chunk (n, 2*j + h).
+// One asynchronous 16-byte global->LDS copy per lane: lane l's data lands at lds_base + 16*l.
+// Written as inline asm so the compiler does not serialise later LDS reads behind it; the caller
+// orders things with wait_async_tiles() + a workgroup barrier.  lds_base must be wave-uniform.
+__device__ __forceinline__ void async_load16(const void* tile_base, int byte_off, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(byte_off), "s"(tile_base) : "memory");
+}
+
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(unsigned long long)(const __attribute__((address_space(3))) char*)p;
+}
+
+// Asynchronous staging of a ROWS x D tile into a PaddedTile.  Each wave instruction fills one
+// 1 KiB slab; a lane's slot maps to (row, chunk) = (slot / CHP, slot % CHP), pad slots are skipped.
+// The per-lane global offsets are computed once (init) because the tile geometry never changes.
+template <typename E, int D, int PAD, int ROWS, int NT>
+struct AsyncPaddedLoader {
+    typedef PaddedTile<E, D, PAD> P;
+    static constexpr int SLOTS = ROWS * P::CHP;
+    static constexpr int SLABS = (SLOTS + 63) / 64;
+    static constexpr int NWV = NT / 64;
+    static constexpr int PER_WAVE = (SLABS + NWV - 1) / NWV;
+    int goff[PER_WAVE];  // byte offset from the tile's first row, -1 for a pad / unused slot
+
+    __device__ __forceinline__ void init(int64_t row_stride, int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            int slot = (i * NWV + wave) * 64 + lane;
+            int row = slot / P::CHP, c = slot % P::CHP;
+            goff[i] = (slot < SLOTS && c < P::CH) ? (int)(row * row_stride * Elem<E>::kBytes) + c * 16 : -1;
+        }
+    }
+
+    // tile_base: global address of the tile's first row (wave-uniform); lds: the tile in LDS.
+    __device__ __forceinline__ void issue(const typename Elem<E>::type* tile_base, int64_t row_stride,
+                                          int rows_valid, char* lds, int wave, int lane) const {
+        const unsigned lds_base = lds_address(lds);
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int slab = i * NWV + wave;
+            if (SLABS % NWV != 0 && slab >= SLABS) continue;
+            if (rows_valid >= ROWS) {
+                if (goff[i] >= 0) async_load16(tile_base, goff[i], lds_base + slab * 1024);
+            } else {
+                // ragged last tile: rows past the end of the tensor read as zeros
+                int slot = slab * 64 + lane;
+                int row = slot / P::CHP, c = slot % P::CHP;
+                if (slot < SLOTS && c < P::CH) {
+                    if (row < rows_valid) {
+                        async_load16(tile_base, goff[i], lds_base + slab * 1024);
+                    } else {
+                        *reinterpret_cast<i32x4*>(lds + slot * 16) = i32x4{0, 0, 0, 0};
+                    }
+                }
+            }
+        }
+    }
+};
+
+// Resident operand: the wave's 32 rows as MFMA B operands in registers,
+// c[j] = the 16-byte chunk (row n, 2*j + h).
 template <typename E, int D>
 struct Resident {
     static constexpr int NJ = LdsTile<E, D>::CH / 2;
@@ -253,15 +329,107 @@ struct Resident {
     i32x4 c[NJ];
 };
 
+// Per-lane byte offsets of everything a wave reads from an LDS tile, computed once per kernel so
+// the inner loops issue LDS reads with no address arithmetic.  Offsets are for the first 32-row
+// block of a tile; block kb adds kb * BLOCK_BYTES (valid when LdsTile::kBlockAffine, otherwise the
+// address is recomputed).
+//   row[j]          16-byte chunk (row n, 2*j + h): the row-wise operand.  For 16-bit types one
+//                   MFMA operand (contraction slots 16*j + 8*h ..), for fp32 four (slots 8*j + 4*h ..).
+//   tr[db][s][w]    16-bit types: address this lane supplies to ds_read_b64_tr_b16 for the transposed
+//                   operand of head-dim block db, 16-row half s, first (w = 0) or second (w = 1)
+//                   group of four contraction rows.
+// ds_read_b64_tr_b16 works on groups of 16 lanes: lane r of a group supplies the address of four
+// consecutive 16-bit elements X[k0 + r/4][n0 + 4*(r%4) ..] and lane i of the group receives
+// X[k0 + 0..3][n0 + i].
 template <typename E, int D>
-__device__ __forceinline__ f32x16 mma_rowwise(const char* lds, int row0, const Resident<E, D>& b,
-                                              f32x16 acc, int lane) {
-    constexpr int NJ = Resident<E, D>::NJ;
-    int n = lane & 31, h = lane >> 5;
+struct OperandOffsets {
+    typedef LdsTile<E, D> L;
+    static constexpr int NJ = L::CH / 2;
+    static constexpr int DB = (D + 31) / 32;
+    int row[NJ];
+    int tr[Elem<E>::k16 ? DB : 1][2][2];
+
+    __device__ __forceinline__ void init(int lane) {
+        const int n = lane & 31, h = lane >> 5;
 #pragma unroll
-    for (int j = 0; j < NJ; j++) {
-        i32x4 a = lds_row_chunk<E, D>(lds, row0 + n, 2 * j + h);
-        acc = Elem<E>::mma(a, b.c[j], acc);
+        for (int j = 0; j < NJ; j++) row[j] = L::chunk_off(n, 2 * j + h);
+        if constexpr (Elem<E>::k16) {
+            const int r = lane & 15, colgrp = (lane >> 4) & 1;
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                int col = 32 * db + 16 * colgrp + 4 * (r & 3);
+                if (D < 32) col &= (D - 1);
+#pragma unroll
+                for (int s = 0; s < 2; s++)
+#pragma unroll
+                    for (int w = 0; w < 2; w++) tr[db][s][w] = L::elem_off(16 * s + 8 * w + 4 * h + (r >> 2), col);
+            }
+        }
+    }
+
+    __device__ __forceinline__ i32x4 row_chunk(const char* lds, int kb, int j, int lane) const {
+        if constexpr (L::kBlockAffine) {
+            return *reinterpret_cast<const i32x4*>(lds + row[j] + kb * L::BLOCK_BYTES);
+        } else {
+            return *reinterpret_cast<const i32x4*>(lds + L::chunk_off(32 * kb + (lane & 31), 2 * j + (lane >> 5)));
+        }
+    }
+
+    // Transposed 16-bit operand: rows {32*kb + 16*s + 4*h + (0..3), + 8} at column 32*db + n.
+    __device__ __forceinline__ i32x4 tr_operand(const char* lds, int kb, int s, int db, int lane) const {
+        int o0, o1;
+        if constexpr (L::kBlockAffine) {
+            o0 = tr[db][s][0] + kb * L::BLOCK_BYTES;
+            o1 = tr[db][s][1] + kb * L::BLOCK_BYTES;
+        } else {
+            const int r = lane & 15, colgrp = (lane >> 4) & 1, h = lane >> 5;
+            int col = 32 * db + 16 * colgrp + 4 * (r & 3);
+            if (D < 32) col &= (D - 1);
+            const int rw = 32 * kb + 16 * s + 4 * h + (r >> 2);
+            o0 = L::elem_off(rw, col);
+            o1 = L::elem_off(rw + 8, col);
+        }
+        i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(lds + o0));
+        i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(lds + o1));
+        i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(i32x4, v);
+    }
+};
+
+// acc(32 rows of the LDS tile x 32 cols) += X[32*kb + 0..31][:] * B^T, B = resident rows.
+template <typename E, int D>
+__device__ __forceinline__ f32x16 mma_rowwise(const char* lds, int kb, const OperandOffsets<E, D>& ofs,
+                                              const Resident<E, D>& b, f32x16 acc, int lane) {
+#pragma unroll
+    for (int j = 0; j < Resident<E, D>::NJ; j++) acc = Elem<E>::mma(ofs.row_chunk(lds, kb, j, lane), b.c[j], acc);
+    return acc;
+}
+
+// acc(32 out-rows x 32 cols) += X^T * P: contraction over the 32 rows of block kb of the LDS tile,
+// P a 32x32 accumulator-layout block (rows = contraction index) reused as B operand, output row
+// index = column 32*db + n of the LDS tile.
+template <typename E, int D>
+__device__ __forceinline__ f32x16 mma_transposed(const char* lds, int kb, int db, const OperandOffsets<E, D>& ofs,
+                                                 f32x16 p, f32x16 acc, int lane) {
+    if constexpr (Elem<E>::k16) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            f32x8 ps;
+#pragma unroll
+            for (int e = 0; e < 8; e++) ps[e] = p[8 * s + e];
+            acc = Elem<E>::mma(ofs.tr_operand(lds, kb, s, db, lane), Elem<E>::pack8(ps), acc);
+        }
+    } else {
+        typedef LdsTile<E, D> L;
+        int h = lane >> 5;
+        int col = 32 * db + (lane & 31);
+        if (D < 32) col &= (D - 1);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            int rw = 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+            float a = *reinterpret_cast<const float*>(lds + L::elem_off(rw, col));
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, p[r], acc, 0, 0, 0);
+        }
     }
     return acc;
 }

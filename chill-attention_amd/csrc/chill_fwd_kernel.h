@@ -5,12 +5,17 @@
 // Each wave owns 32 query rows.  It keeps Q^T as MFMA B operands in registers and computes the
 // TRANSPOSED score block S^T = K Q^T, so that in the accumulator layout one lane holds scores of
 // a single query row: the running max / sum of the online softmax (chill_fwd.py:214-226) are
-// per-lane scalars, and the only cross-lane step is one v_permlane32_swap per tile.  P^T in
+// per-lane scalars, and the only cross-lane step is one v_permlane32_swap per block.  P^T in
 // accumulator layout is directly the B operand of O^T += V^T P^T; V^T comes out of LDS through
-// the transposing read (ds_read_b64_tr_b16), so V is staged exactly like K.
+// the transposing read (ds_read_b64_tr_b16), so V is staged in its natural row-major form.
 //
-// K/V tiles are staged through double-buffered, XOR-swizzled LDS by the whole workgroup; the
-// global loads of tile i+1 are in flight while tile i is consumed.
+// K/V tiles are staged by the whole workgroup through a ring of padded LDS stages filled by
+// asynchronous global->LDS loads: while tile i is consumed, tile i+1 is already resident and
+// tile i+2 is in flight.  Work proceeds in steps of 32 keys, software-pipelined: the score MFMAs of
+// step t+1 are issued before the softmax of step t, so matrix and vector units overlap in a wave.
+//
+// The softmax rescales lazily: a row's reference max is raised (and O, l rescaled) only when a
+// block max exceeds it by more than kRescaleTau, a wave-uniform rare branch.
 //
 // Tile skipping and the predicate-free path follow chill_fwd.py:131-139 and :161-185, evaluated
 // per WAVE (32 rows): a wave skips streamed tiles outside its own k-range and drops the predicate
@@ -23,16 +28,33 @@
 
 namespace chill {
 
-template <typename E, int D, int MASK, int NW, int TK>
+// Lazy-rescale threshold of the online softmax, in log2 units: P stays below 2^kRescaleTau.
+constexpr float kRescaleTau = 8.0f;
+
+template <typename E, int D, int TK>
+struct FwdLds {
+    typedef PaddedTile<E, D, rowwise_pad<E, D>()> KT;
+    typedef PaddedTile<E, D, transposed_pad<E, D>()> VT;
+    static constexpr int K_BYTES = KT::bytes(TK);
+    static constexpr int V_BYTES = VT::bytes(TK);
+    static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
+};
+
+template <typename E, int D, int MASK, int NW, int TK, int NS>
 __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
                                                       int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     using M = Mask<MASK>;
+    typedef FwdLds<E, D, TK> Lds;
+    typedef typename Lds::KT KT;
+    typedef typename Lds::VT VT;
     constexpr int TQ = NW * 32;
     constexpr int NT = NW * 64;
-    constexpr int KB = TK / 32;         // 32-key blocks per streamed tile
+    constexpr int KB = TK / 32;         // 32-key blocks ("steps") per streamed tile
     constexpr int DB = (D + 31) / 32;   // 32-wide blocks of the head dim
-    constexpr int TILE_BYTES = LdsTile<E, D>::bytes(TK);
+    constexpr int NJ = KT::CH / 2;      // 16-byte chunk pairs along the head dim
+    constexpr int LA = NS - 2;          // tiles certified resident ahead of the one being consumed
+    static_assert(NS == 2 || NS == 3, "two or three LDS stages");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
@@ -46,7 +68,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;
     const int h = lane >> 5;
 
@@ -70,101 +92,180 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
     const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
     const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
 
+    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
+    const int n_tiles = wg.end - wg.start;
+    AsyncPaddedLoader<E, D, rowwise_pad<E, D>(), TK, NT> load_k;
+    AsyncPaddedLoader<E, D, transposed_pad<E, D>(), TK, NT> load_v;
+    load_k.init(p.sk.t, wave, lane);
+    load_v.init(p.sv.t, wave, lane);
+    auto issue_tile = [&](int i, int st_index) {
+        int k0 = (wg.start + i) * TK;
+        char* st = smem + st_index * Lds::STAGE_BYTES;
+        load_k.issue(kptr + (int64_t)k0 * p.sk.t, p.sk.t, p.T - k0, st, wave, lane);
+        load_v.issue(vptr + (int64_t)k0 * p.sv.t, p.sv.t, p.T - k0, st + Lds::K_BYTES, wave, lane);
+    };
+#pragma unroll
+    for (int i = 0; i <= LA; i++)
+        if (i < n_tiles) issue_tile(i, i);
+
     const int qw = qb + 32 * wave;
     Resident<E, D> qf;
     load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
 
-    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
-    TileRange wr = {0, 0, 0, 0};
+    TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
+    // this wave's tiles, as offsets into the workgroup's ring
+    const int ta = wr.start - wg.start, tb = wr.end - wg.start;
+    const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
+
+    // per-lane LDS offsets inside a stage; everything else is an immediate
+    const int k_lane = n * KT::PITCH + h * 16;
+    int v_lane;
+    if constexpr (Elem<E>::k16) {
+        const int r = lane & 15, colgrp = (lane >> 4) & 1;
+        int col = 16 * colgrp + 4 * (r & 3);
+        if (D < 32) col &= (D - 1);
+        v_lane = Lds::K_BYTES + (4 * h + (r >> 2)) * VT::PITCH + col * 2;
+    } else {
+        v_lane = Lds::K_BYTES + 4 * h * VT::PITCH + (D < 32 ? (n & (D - 1)) : n) * 4;
+    }
 
     f32x16 o[DB];
 #pragma unroll
     for (int i = 0; i < DB; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[i][r] = 0.f;
-    float m_run = -INFINITY;
-    float l_run = 0.f;
+    float m_run = -INFINITY;  // reference max of the row (scaled, log2 domain)
+    float m_use = 0.f;        // m_run, or 0 while the row has seen no unmasked key
+    float l_run = 0.f;        // this lane's share of the row sum
     const int q_pos = qw + n;
-    const float scale = p.scale_log2;
+    const bool negate = p.scale_log2 < 0.f;  // max(scale * s) = |scale| * max(sign * s)
+    const float scale = negate ? -p.scale_log2 : p.scale_log2;
 
-    TileStager<E, D, TK, NT> stage_k, stage_v;
-    {
-        int k0 = wg.start * TK;
-        stage_k.fetch(kptr + (int64_t)k0 * p.sk.t, p.sk.t, p.T - k0, tid);
-        stage_v.fetch(vptr + (int64_t)k0 * p.sv.t, p.sv.t, p.T - k0, tid);
-    }
-
-    for (int kt = wg.start; kt < wg.end; kt++) {
-        char* lds_k = smem + ((kt - wg.start) & 1) * 2 * TILE_BYTES;
-        char* lds_v = lds_k + TILE_BYTES;
-        stage_k.commit(lds_k, tid);
-        stage_v.commit(lds_v, tid);
-        __syncthreads();
-        if (kt + 1 < wg.end) {
-            int k1 = (kt + 1) * TK;
-            stage_k.fetch(kptr + (int64_t)k1 * p.sk.t, p.sk.t, p.T - k1, tid);
-            stage_v.fetch(vptr + (int64_t)k1 * p.sv.t, p.sv.t, p.T - k1, tid);
+    // S^T block of step kb of the tile at LDS address `stage`:  K[32*kb + 0..31][:] Q^T
+    auto scores = [&](f32x16& dst, const lds_char* stage, int kb) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) dst[r] = 0.f;
+        const lds_char* base = stage + k_lane + kb * 32 * KT::PITCH;
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+            dst = Elem<E>::mma(*reinterpret_cast<const lds_i32x4*>(base + j * 32), qf.c[j], dst);
+    };
+    // sign, mask and block max (scaled) of a score block
+    auto prepare = [&](f32x16& sc, bool full, int key0) -> float {
+        if (negate) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) sc[r] = -sc[r];
         }
-        if (kt < wr.start || kt >= wr.end) continue;
-        const bool full = (kt >= wr.full_start) && (kt < wr.full_end);
-        const int k0 = kt * TK;
-
-        // S^T = K Q^T
-        f32x16 s[KB];
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
-            s[kb] = mma_rowwise<E, D>(lds_k, 32 * kb, qf, s[kb], lane);
-        }
-
-        float mx = -INFINITY;
-        if (full) {
-#pragma unroll
-            for (int kb = 0; kb < KB; kb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    s[kb][r] *= scale;
-                    mx = fmaxf(mx, s[kb][r]);
-                }
-        } else {
-#pragma unroll
-            for (int kb = 0; kb < KB; kb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    int key = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
-                    bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
-                    s[kb][r] = ok ? s[kb][r] * scale : -INFINITY;
-                    mx = fmaxf(mx, s[kb][r]);
-                }
-        }
-        mx = max_across_halves(mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run - m_safe);
-        float psum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++)
+        if (!full) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                float pv = fast_exp2(s[kb][r] - m_safe);
-                s[kb][r] = pv;
+                int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+                bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
+                sc[r] = ok ? sc[r] : -INFINITY;
+            }
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
+        return max_across_halves(mx) * scale;
+    };
+    // O^T += V^T P^T for step kb of the tile at `stage`
+    auto accumulate = [&](const f32x16& pr, const lds_char* stage, int kb) {
+        const lds_char* base = stage + v_lane + kb * 32 * VT::PITCH;
+        if constexpr (Elem<E>::k16) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                f32x8 ps;
+#pragma unroll
+                for (int e = 0; e < 8; e++) ps[e] = pr[8 * s2 + e];
+                const i32x4 bop = Elem<E>::pack8(ps);
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    const lds_char* a0 = base + (16 * s2) * VT::PITCH + db * 64;
+                    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)a0);
+                    i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(a0 + 8 * VT::PITCH));
+                    i16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = Elem<E>::mma(__builtin_bit_cast(i32x4, av), bop, o[db]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    float a = *reinterpret_cast<const lds_float*>(base + (8 * (r / 4) + (r % 4)) * VT::PITCH + db * 128);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, pr[r], o[db], 0, 0, 0);
+                }
+        }
+    };
+
+    f32x16 s[2];         // scores of the current and of the next step
+    float mx_cur = 0.f;  // block max of s[current], already scaled
+    const lds_char* lds0 = (const lds_char*)smem;
+    // Q must have arrived before the loop: inside it the only vector-memory traffic is the async
+    // tile loads, and the compiler must not place a wait for them in front of the first MFMA
+#pragma unroll
+    for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(qf.c[j]));
+
+    int st_cur = NS - 1;  // LDS stage of tile i (advanced at the top of the loop)
+    int st_issue = LA;    // LDS stage the next issued tile goes to
+    for (int i = 0; i < n_tiles; i++) {
+        // tiles <= i + LA have landed for every wave, and everyone is done with tile i - 1
+        wait_async_tiles();
+        __syncthreads();
+        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        if (i + LA + 1 < n_tiles) issue_tile(i + LA + 1, st_issue);
+        if (i < ta || i >= tb) continue;
+        const lds_char* stage = lds0 + st_cur * Lds::STAGE_BYTES;
+        const lds_char* stage_next = lds0 + (st_cur + 1 == NS ? 0 : st_cur + 1) * Lds::STAGE_BYTES;
+        const bool full = (i >= fa) && (i < fb);
+        const bool full_next = (i + 1 >= fa) && (i + 1 < fb);
+        const int k0 = (wg.start + i) * TK;
+        if (LA == 0 || i == ta) {
+            scores(s[0], stage, 0);
+            mx_cur = prepare(s[0], full, k0);
+        }
+
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+            f32x16& cur = s[kb & 1];
+            f32x16& nxt = s[(kb + 1) & 1];
+            // rare path: raise the reference max and rescale what has been accumulated
+            const bool raise = mx_cur > m_run + kRescaleTau;
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+                const float m_new = raise ? mx_cur : m_run;
+                const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = fast_exp2(m_use - m_use_new);
+                m_run = m_new;
+                m_use = m_use_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; db++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+            }
+            // scores of the next step fly while this step's softmax runs
+            const bool in_tile = kb + 1 < KB;
+            const bool have_next = in_tile || (LA >= 1 && i + 1 < tb);
+            if (in_tile) {
+                scores(nxt, stage, kb + 1);
+            } else if (LA >= 1 && i + 1 < tb) {
+                scores(nxt, stage_next, 0);
+            }
+            float psum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float pv = fast_exp2(__builtin_fmaf(cur[r], scale, -m_use));
+                cur[r] = pv;
                 psum += pv;
             }
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
-#pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) o[db][r] *= alpha;
-
-        // O^T += V^T P^T
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++)
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-                o[db] = mma_transposed<E, D>(lds_v, 32 * kb, 32 * db, s[kb], o[db], lane);
+            l_run += psum;
+            accumulate(cur, stage, kb);
+            if (have_next) mx_cur = in_tile ? prepare(nxt, full, k0 + 32 * (kb + 1)) : prepare(nxt, full_next, k0 + TK);
+        }
+        if (KB & 1) s[0] = s[1];  // odd step count: the prefetched scores sit in the other buffer
     }
 
     // epilogue: O = acc / l, LSE2 = m + log2(l) (chill_fwd.py:288-289, 327-328)
@@ -184,16 +285,22 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
 // from the static table.
 template <typename E, int D>
 int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
+    // the async loader keeps per-lane global offsets in 32 bits
+    const int64_t max_stride = p.sk.t > p.sv.t ? p.sk.t : p.sv.t;
+    if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = fwd_tile_config(MASK_ID, D, Elem<E>::kDType);
         static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+        constexpr int NS = fwd_stages_for(cfg.streamed, D, Elem<E>::kDType);
+        static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES,
+                      "table and kernel disagree on LDS");
         const int n_q_tiles = cdiv(p.T, cfg.rows);
         const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        auto kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed>;
+        auto kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
         const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

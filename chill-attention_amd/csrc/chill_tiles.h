@@ -14,13 +14,27 @@ namespace chill {
 
 constexpr int elem_bytes(int dtype) { return dtype == CHILL_F32 ? 4 : 2; }
 
+// Forward LDS stage: a K tile padded for row-wise reads and a V tile padded for transposed reads
+// (pads as in PaddedTile, chill_device.h).
+constexpr int fwd_stage_bytes(int streamed, int D, int dtype) {
+    const int rb = D * elem_bytes(dtype);
+    const int vpad = dtype == CHILL_F32 ? 32 : (rb >= 128 ? 64 : 0);
+    return streamed * (rb + 16) + streamed * (rb + vpad);
+}
+
+// LDS stages of the forward K/V ring: three (one tile resident ahead, one in flight) when they fit
+// in 144 KiB, else two.
+constexpr int fwd_stages_for(int streamed, int D, int dtype) {
+    return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
+}
+
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
     const int waves = fast16 ? 8 : 4;
     const int streamed = fast16 ? 64 : 32;
-    // double-buffered K and V tiles
-    return TileConfig{waves * 32, streamed, waves, 2 * 2 * streamed * D * elem_bytes(dtype)};
+    return TileConfig{waves * 32, streamed, waves,
+                      fwd_stages_for(streamed, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
 }
 
 constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
