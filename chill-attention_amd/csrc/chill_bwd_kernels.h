@@ -75,7 +75,9 @@ int launch_delta(const DeltaParams& p, hipStream_t stream) {
 }
 
 // Probabilities and score gradients of one 32x32 block, in place: on entry s = raw scores,
-// dp = dO.V products; on exit s = P (0 where masked), dp = dS = P * (dP - delta).
+// dp = dO.V products; on exit s = P (0 where masked), dp = dS = P * (dP - delta).  A row that saw
+// no key has LSE2 = -inf and P = exp2(+inf) = inf there; such a row can only occur in blocks that
+// take the predicate path, whose select (not a multiply) turns it into 0.
 // Row/column meaning differs between the two kernels, so the caller supplies, per accumulator
 // register r, the LSE2 / delta of the query and the (q, k) positions.
 template <int MASK, bool PARTIAL, typename PosFn>
@@ -97,7 +99,9 @@ __device__ __forceinline__ void softmax_grad_block(f32x16& s, f32x16& dp, float 
 }
 
 // ------------------------------------------------------------------------------------------ dQ
-template <typename E, int D, int MASK, int NW, int TK>
+// Same skeleton as the forward kernel: asynchronous K/V ring, 32-key steps, the two score GEMMs of
+// step t+1 (S^T and dP^T) issued before the vector work of step t.
+template <typename E, int D, int MASK, int NW, int TK, int NS>
 __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
                                                      int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
@@ -105,7 +109,11 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
     constexpr int NT = NW * 64;
     constexpr int KB = TK / 32;
     constexpr int DB = (D + 31) / 32;
+    constexpr int NJ = Resident<E, D>::NJ;
     constexpr int TILE_BYTES = LdsTile<E, D>::bytes(TK);
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K tile, then V tile
+    constexpr int LA = NS - 2;
+    static_assert(NS == 2 || NS == 3, "two or three LDS stages");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
@@ -118,7 +126,7 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;
     const int h = lane >> 5;
 
@@ -137,6 +145,21 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
     const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
     const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
 
+    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
+    const int n_tiles = wg.end - wg.start;
+    AsyncSwizzledLoader<E, D, TK, NT> load_k, load_v;
+    load_k.init(p.sk.t, wave, lane);
+    load_v.init(p.sv.t, wave, lane);
+    auto issue_tile = [&](int i, int st_index) {
+        int k0 = (wg.start + i) * TK;
+        char* st = smem + st_index * STAGE_BYTES;
+        load_k.issue(kptr + (int64_t)k0 * p.sk.t, p.T - k0, st, wave, lane);
+        load_v.issue(vptr + (int64_t)k0 * p.sv.t, p.T - k0, st + TILE_BYTES, wave, lane);
+    };
+#pragma unroll
+    for (int i = 0; i <= LA; i++)
+        if (i < n_tiles) issue_tile(i, i);
+
     const int qw = qb + 32 * wave;
     const int q_pos = qw + n;
     OperandOffsets<E, D> ofs;
@@ -149,11 +172,11 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
         lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
         delta_q = p.delta[b * p.delta_b + hd * p.delta_h + q_pos];
     }
-    if (lse_q == -INFINITY) lse_q = 0.f;  // fully masked row: P is forced to 0 by the predicate
 
-    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
-    TileRange wr = {0, 0, 0, 0};
+    TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
+    const int ta = wr.start - wg.start, tb = wr.end - wg.start;
+    const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
 
     f32x16 dq[DB];
 #pragma unroll
@@ -162,38 +185,49 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
         for (int r = 0; r < 16; r++) dq[i][r] = 0.f;
     const float scale = p.scale_log2;
 
-    TileStager<E, D, TK, NT> stage_k, stage_v;
-    {
-        int k0 = wg.start * TK;
-        stage_k.fetch(kptr + (int64_t)k0 * p.sk.t, p.sk.t, p.T - k0, tid);
-        stage_v.fetch(vptr + (int64_t)k0 * p.sv.t, p.sv.t, p.T - k0, tid);
-    }
-
-    for (int kt = wg.start; kt < wg.end; kt++) {
-        char* lds_k = smem + ((kt - wg.start) & 1) * 2 * TILE_BYTES;
-        char* lds_v = lds_k + TILE_BYTES;
-        stage_k.commit(lds_k, tid);
-        stage_v.commit(lds_v, tid);
-        __syncthreads();
-        if (kt + 1 < wg.end) {
-            int k1 = (kt + 1) * TK;
-            stage_k.fetch(kptr + (int64_t)k1 * p.sk.t, p.sk.t, p.T - k1, tid);
-            stage_v.fetch(vptr + (int64_t)k1 * p.sv.t, p.sv.t, p.T - k1, tid);
+    // S^T = K Q^T and dP^T = V dO^T of step kb of the stage at `stage`
+    auto gemms = [&](f32x16& sdst, f32x16& dpdst, const lds_char* stage, int kb) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            sdst[r] = 0.f;
+            dpdst[r] = 0.f;
         }
-        if (kt < wr.start || kt >= wr.end) continue;
-        const bool full = (kt >= wr.full_start) && (kt < wr.full_end);
-        const int k0 = kt * TK;
+        sdst = mma_rowwise<E, D>(stage, kb, ofs, qf, sdst, lane);
+        dpdst = mma_rowwise<E, D>(stage + TILE_BYTES, kb, ofs, dof, dpdst, lane);
+    };
+
+    f32x16 s[2], dp[2];
+    const lds_char* lds0 = (const lds_char*)smem;
+    // the resident operands must have arrived before the loop, where the only vector-memory traffic
+    // is the async tile loads and no compiler-placed wait may cover them
+#pragma unroll
+    for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(qf.c[j]), "v"(dof.c[j]));
+    asm volatile("" ::"v"(lse_q), "v"(delta_q));
+
+    int st_cur = NS - 1;
+    int st_issue = LA;
+    for (int i = 0; i < n_tiles; i++) {
+        wait_async_tiles();
+        __syncthreads();
+        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        if (i + LA + 1 < n_tiles) issue_tile(i + LA + 1, st_issue);
+        if (i < ta || i >= tb) continue;
+        const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
+        const lds_char* stage_next = lds0 + (st_cur + 1 == NS ? 0 : st_cur + 1) * STAGE_BYTES;
+        const bool full = (i >= fa) && (i < fb);
+        const int k0 = (wg.start + i) * TK;
+        if (LA == 0 || i == ta) gemms(s[0], dp[0], stage, 0);
 
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
-            f32x16 s, dp;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                s[r] = 0.f;
-                dp[r] = 0.f;
+            f32x16& cs = s[kb & 1];
+            f32x16& cdp = dp[kb & 1];
+            if (kb + 1 < KB) {
+                gemms(s[(kb + 1) & 1], dp[(kb + 1) & 1], stage, kb + 1);
+            } else if (LA >= 1 && i + 1 < tb) {
+                gemms(s[(kb + 1) & 1], dp[(kb + 1) & 1], stage_next, 0);
             }
-            s = mma_rowwise<E, D>(lds_k, kb, ofs, qf, s, lane);
-            dp = mma_rowwise<E, D>(lds_v, kb, ofs, dof, dp, lane);
             auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
                 q = q_pos;
                 k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
@@ -201,12 +235,15 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
                 delta = delta_q;
             };
             if (full)
-                softmax_grad_block<MASK, false>(s, dp, scale, seq_len, p.margs, pos);
+                softmax_grad_block<MASK, false>(cs, cdp, scale, seq_len, p.margs, pos);
             else
-                softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-                dq[db] = mma_transposed<E, D>(lds_k, kb, db, ofs, dp, dq[db], lane);
+                softmax_grad_block<MASK, true>(cs, cdp, scale, seq_len, p.margs, pos);
+            // dQ^T += K^T dS^T
+            mma_transposed<E, D>(stage, kb, ofs, cdp, dq, lane);
+        }
+        if (KB & 1) {
+            s[0] = s[1];
+            dp[0] = dp[1];
         }
     }
 
@@ -216,16 +253,19 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
 
 template <typename E, int D>
 int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
+    const int64_t max_stride = p.sk.t > p.sv.t ? p.sk.t : p.sv.t;
+    if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = dq_tile_config(MASK_ID, D, Elem<E>::kDType);
         static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+        constexpr int NS = dq_stages_for(cfg.streamed, D, Elem<E>::kDType);
         const int n_q_tiles = cdiv(p.T, cfg.rows);
         const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        auto kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed>;
+        auto kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
         const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -239,7 +279,11 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
-template <typename E, int D, int MASK, int NW, int TQS>
+// Resident: 32 key rows per wave (K, V as B operands).  Streamed through the LDS ring: Q and dO
+// tiles of TQS query rows with their LSE2 / delta, for every query head of the GQA group in turn
+// (chill_bwd_dkdv.py:156).  Steps of 32 queries; S and dP of step t+1 are issued before the vector
+// work of step t.
+template <typename E, int D, int MASK, int NW, int TQS, int NS>
 __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
                                                        int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
@@ -247,9 +291,13 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
     constexpr int NT = NW * 64;
     constexpr int QB = TQS / 32;
     constexpr int DB = (D + 31) / 32;
+    constexpr int NJ = Resident<E, D>::NJ;
     constexpr int TILE_BYTES = LdsTile<E, D>::bytes(TQS);
-    constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * TQS * 4;
-    static_assert(NT >= 2 * TQS, "LSE2 / delta staging needs one thread per value");
+    constexpr int VEC_BYTES = TQS * 4;
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * VEC_BYTES;  // Q, dO, LSE2, delta
+    constexpr int LA = NS - 2;
+    static_assert(NS == 2 || NS == 3, "two or three LDS stages");
+    static_assert(TQS <= 64, "one wave instruction stages a vector");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
@@ -262,7 +310,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;
     const int h = lane >> 5;
 
@@ -279,6 +327,43 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         return;
     }
 
+    const TileRange wg = tile_range<MASK, false>(kb0, TKR, TQS, seq_len, false, p.margs);
+    const int n_tiles = wg.end - wg.start;
+    const int n_iters = n_tiles * p.group;
+
+    AsyncSwizzledLoader<E, D, TQS, NT> load_q, load_do;
+    load_q.init(p.sq.t, wave, lane);
+    load_do.init(p.sdo.t, wave, lane);
+    // iteration it = (group head g, q-tile): stage it % NS
+    auto issue_iter = [&](int it, int st_index) {
+        const int g = it / n_tiles;
+        const int q0 = (wg.start + it % n_tiles) * TQS;
+        const int hq = hkv * p.group + g;
+        char* st = smem + st_index * STAGE_BYTES;
+        const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
+        const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
+        load_q.issue(qptr + (int64_t)q0 * p.sq.t, p.T - q0, st, wave, lane);
+        load_do.issue(doptr + (int64_t)q0 * p.sdo.t, p.T - q0, st + TILE_BYTES, wave, lane);
+        if (wave == 0) {
+            // LSE2 and delta of the tile's rows; rows past the end of the tensor read as zero
+            const float* lse = p.lse + b * p.lse_b + hq * p.lse_h + q0;
+            const float* del = p.delta + b * p.delta_b + hq * p.delta_h + q0;
+            char* vec = st + 2 * TILE_BYTES;
+            if (lane < TQS) {
+                if (q0 + lane < p.T) {
+                    async_load4(lse, lane * 4, lds_address(vec));
+                    async_load4(del, lane * 4, lds_address(vec + VEC_BYTES));
+                } else {
+                    reinterpret_cast<float*>(vec)[lane] = 0.f;
+                    reinterpret_cast<float*>(vec + VEC_BYTES)[lane] = 0.f;
+                }
+            }
+        }
+    };
+#pragma unroll
+    for (int i = 0; i <= LA; i++)
+        if (i < n_iters) issue_iter(i, i);
+
     const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
     const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
     const int kw = kb0 + 32 * wave;
@@ -289,9 +374,10 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
     load_resident<E, D>(kf, kptr + (int64_t)kw * p.sk.t, p.sk.t, p.T - kw, lane);
     load_resident<E, D>(vf, vptr + (int64_t)kw * p.sv.t, p.sv.t, p.T - kw, lane);
 
-    const TileRange wg = tile_range<MASK, false>(kb0, TKR, TQS, seq_len, false, p.margs);
-    TileRange wr = {0, 0, 0, 0};
+    TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (kw < seq_len) wr = tile_range<MASK, false>(kw, 32, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
+    const int ta = wr.start - wg.start, tb = wr.end - wg.start;
+    const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
 
     f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -303,64 +389,62 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         }
     const float scale = p.scale_log2;
 
-    const int n_tiles = wg.end - wg.start;
-    const int n_iters = n_tiles * p.group;
-
-    TileStager<E, D, TQS, NT> stage_q, stage_do;
-    float stage_vec = 0.f;  // thread tid < TQS stages LSE2[tid], TQS <= tid < 2*TQS stages delta
-    auto fetch = [&](int it) {
-        int g = it / n_tiles;
-        int qt = wg.start + it % n_tiles;
-        int hq = hkv * p.group + g;
-        int q0 = qt * TQS;
-        const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
-        const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
-        stage_q.fetch(qptr + (int64_t)q0 * p.sq.t, p.sq.t, p.T - q0, tid);
-        stage_do.fetch(doptr + (int64_t)q0 * p.sdo.t, p.sdo.t, p.T - q0, tid);
-        stage_vec = 0.f;
-        if (tid < 2 * TQS) {
-            int qi = q0 + (tid % TQS);
-            if (qi < p.T) {
-                if (tid < TQS) {
-                    float v = p.lse[b * p.lse_b + hq * p.lse_h + qi];
-                    stage_vec = (v == -INFINITY) ? 0.f : v;
-                } else {
-                    stage_vec = p.delta[b * p.delta_b + hq * p.delta_h + qi];
-                }
-            }
+    // S = Q K^T and dP = dO V^T of step qb of the stage at `stage`
+    auto gemms = [&](f32x16& sdst, f32x16& dpdst, const lds_char* stage, int qb) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            sdst[r] = 0.f;
+            dpdst[r] = 0.f;
         }
+        sdst = mma_rowwise<E, D>(stage, qb, ofs, kf, sdst, lane);
+        dpdst = mma_rowwise<E, D>(stage + TILE_BYTES, qb, ofs, vf, dpdst, lane);
     };
-    if (n_iters > 0) fetch(0);
 
+    f32x16 s[2], dp[2];
+    const lds_char* lds0 = (const lds_char*)smem;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(kf.c[j]), "v"(vf.c[j]));
+
+    int st_cur = NS - 1;
+    int st_issue = LA;
+    int tile = -1;  // position of iteration `it` inside the q-tile range (it % n_tiles)
+    bool have_cur = false;  // s[0] / dp[0] already hold the first step of this iteration
     for (int it = 0; it < n_iters; it++) {
-        char* lds_q = smem + (it & 1) * STAGE_BYTES;
-        char* lds_do = lds_q + TILE_BYTES;
-        float* lds_vec = reinterpret_cast<float*>(lds_do + TILE_BYTES);  // [0,TQS) LSE2, [TQS,2TQS) delta
-        stage_q.commit(lds_q, tid);
-        stage_do.commit(lds_do, tid);
-        if (tid < 2 * TQS) lds_vec[tid] = stage_vec;
+        wait_async_tiles();
         __syncthreads();
-        if (it + 1 < n_iters) fetch(it + 1);
-        const int qt = wg.start + it % n_tiles;
-        if (qt < wr.start || qt >= wr.end) continue;
-        const bool full = (qt >= wr.full_start) && (qt < wr.full_end);
-        const int q0 = qt * TQS;
+        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        tile = tile + 1 == n_tiles ? 0 : tile + 1;
+        if (it + LA + 1 < n_iters) issue_iter(it + LA + 1, st_issue);
+        if (tile < ta || tile >= tb) {
+            have_cur = false;
+            continue;
+        }
+        const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
+        const lds_char* stage_next = lds0 + (st_cur + 1 == NS ? 0 : st_cur + 1) * STAGE_BYTES;
+        const lds_float* vec = reinterpret_cast<const lds_float*>(stage + 2 * TILE_BYTES);
+        const bool full = (tile >= fa) && (tile < fb);
+        const int q0 = (wg.start + tile) * TQS;
+        // the next iteration is one of mine if it is the next tile of my range, or the first tile
+        // of my range for the next head of the group
+        const int tile_next = tile + 1 == n_tiles ? 0 : tile + 1;
+        const bool next_mine = (it + 1 < n_iters) && tile_next >= ta && tile_next < tb;
+        if (!have_cur) gemms(s[0], dp[0], stage, 0);
 
 #pragma unroll
         for (int qb = 0; qb < QB; qb++) {
-            f32x16 s, dp;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                s[r] = 0.f;
-                dp[r] = 0.f;
+            f32x16& cs = s[qb & 1];
+            f32x16& cdp = dp[qb & 1];
+            if (qb + 1 < QB) {
+                gemms(s[(qb + 1) & 1], dp[(qb + 1) & 1], stage, qb + 1);
+            } else if (LA >= 1 && next_mine) {
+                gemms(s[(qb + 1) & 1], dp[(qb + 1) & 1], stage_next, 0);
             }
-            s = mma_rowwise<E, D>(lds_q, qb, ofs, kf, s, lane);
-            dp = mma_rowwise<E, D>(lds_do, qb, ofs, vf, dp, lane);
             f32x4 lse4[4], del4[4];
 #pragma unroll
             for (int g4 = 0; g4 < 4; g4++) {
-                lse4[g4] = *reinterpret_cast<const f32x4*>(lds_vec + 32 * qb + 8 * g4 + 4 * h);
-                del4[g4] = *reinterpret_cast<const f32x4*>(lds_vec + TQS + 32 * qb + 8 * g4 + 4 * h);
+                lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 32 * qb + 8 * g4 + 4 * h);
+                del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 32 * qb + 8 * g4 + 4 * h);
             }
             auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
                 q = q0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
@@ -369,14 +453,16 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
                 delta = del4[r / 4][r % 4];
             };
             if (full)
-                softmax_grad_block<MASK, false>(s, dp, scale, seq_len, p.margs, pos);
+                softmax_grad_block<MASK, false>(cs, cdp, scale, seq_len, p.margs, pos);
             else
-                softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                dv[db] = mma_transposed<E, D>(lds_do, qb, db, ofs, s, dv[db], lane);
-                dk[db] = mma_transposed<E, D>(lds_q, qb, db, ofs, dp, dk[db], lane);
-            }
+                softmax_grad_block<MASK, true>(cs, cdp, scale, seq_len, p.margs, pos);
+            mma_transposed<E, D>(stage + TILE_BYTES, qb, ofs, cs, dv, lane);  // dV^T += dO^T P
+            mma_transposed<E, D>(stage, qb, ofs, cdp, dk, lane);              // dK^T += Q^T dS
+        }
+        have_cur = LA >= 1 && next_mine;
+        if ((QB & 1) && have_cur) {
+            s[0] = s[1];
+            dp[0] = dp[1];
         }
     }
 
@@ -389,16 +475,19 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
 
 template <typename E, int D>
 int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
+    const int64_t max_stride = p.sq.t > p.sdo.t ? p.sq.t : p.sdo.t;
+    if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType);
         static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+        constexpr int NS = dkdv_stages_for(cfg.streamed, D, Elem<E>::kDType);
         const int n_k_tiles = cdiv(p.T, cfg.rows);
         const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        auto kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed>;
+        auto kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
         // mask rule order is (q tile, k tile): the streamed tile is the q tile here
         const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, 32, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {

@@ -195,35 +195,61 @@ struct TileStager {
     }
 };
 
-// Asynchronous staging of a ROWS x D tile straight into LDS (global_load_lds_dwordx4): no
-// registers, no ds_write.  One wave instruction fills a 1 KiB slab: lane l's 16 bytes land at
-// slab base + 16*l, so the lane FETCHES the logical chunk whose swizzled position is its slot.
-// Rows >= rows_valid are zero-filled with ordinary LDS stores.  The caller waits with
-// wait_async_tiles() and then a workgroup barrier before anyone reads the tile.
+// One asynchronous 16-byte global->LDS copy per lane: lane l's data lands at lds_base + 16*l.
+// Written as inline asm so the compiler does not serialise later LDS reads behind it; the caller
+// orders things with wait_async_tiles() + a workgroup barrier.  lds_base must be wave-uniform.
+__device__ __forceinline__ void async_load16(const void* tile_base, int byte_off, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(byte_off), "s"(tile_base) : "memory");
+}
+
+// Same for one 4-byte value per lane (lane l's value lands at lds_base + 4*l).
+__device__ __forceinline__ void async_load4(const void* base, int byte_off, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(lds_base), "v"(byte_off), "s"(base) : "memory");
+}
+
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return (unsigned)(unsigned long long)(const __attribute__((address_space(3))) char*)p;
+}
+
+// Asynchronous staging of a ROWS x D tile into a swizzled LdsTile (tiles that are read both
+// row-wise and transposed).  One wave instruction fills a 1 KiB slab: lane l's 16 bytes land at
+// slab base + 16*l, so the lane FETCHES the logical chunk whose swizzled position is its slot (the
+// swizzle is an involution).  Rows >= rows_valid are zero-filled with ordinary LDS stores.  The
+// caller waits with wait_async_tiles() and then a workgroup barrier before anyone reads the tile.
 template <typename E, int D, int ROWS, int NT>
-struct AsyncTile {
+struct AsyncSwizzledLoader {
     typedef LdsTile<E, D> L;
-    static constexpr int TOTAL = ROWS * L::CH;  // chunks, a multiple of 64
-    static constexpr int SLABS = TOTAL / 64;
+    static constexpr int SLOTS = ROWS * L::CH;  // a multiple of 64
+    static constexpr int SLABS = SLOTS / 64;
     static constexpr int NWV = NT / 64;
     static constexpr int PER_WAVE = (SLABS + NWV - 1) / NWV;
-    static_assert(TOTAL % 64 == 0, "tile must be a whole number of 1 KiB slabs");
+    static_assert(SLOTS % 64 == 0, "tile must be a whole number of 1 KiB slabs");
+    int goff[PER_WAVE];  // byte offset of this lane's chunk from the tile's first row
 
-    __device__ __forceinline__ static void issue(const typename Elem<E>::type* base, int64_t row_stride,
-                                                 int rows_valid, char* lds, int wave, int lane) {
+    __device__ __forceinline__ void init(int64_t row_stride, int wave, int lane) {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; i++) {
-            int slab = i * NWV + wave;
-            if (SLABS % NWV == 0 || slab < SLABS) {
+            int lg = L::phys((i * NWV + wave) * 64 + lane);
+            goff[i] = (int)((lg / L::CH) * row_stride * Elem<E>::kBytes) + (lg % L::CH) * 16;
+        }
+    }
+
+    __device__ __forceinline__ void issue(const typename Elem<E>::type* tile_base, int rows_valid, char* lds,
+                                          int wave, int lane) const {
+        const unsigned lds_base = lds_address(lds);
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int slab = i * NWV + wave;
+            if (SLABS % NWV != 0 && slab >= SLABS) continue;
+            if (rows_valid >= ROWS) {
+                async_load16(tile_base, goff[i], lds_base + slab * 1024);
+            } else {
                 int slot = slab * 64 + lane;
-                int lg = L::phys(slot);  // the swizzle is an involution
-                int row = lg / L::CH;
-                int c = lg % L::CH;
+                int row = L::phys(slot) / L::CH;
                 if (row < rows_valid) {
-                    const char* g = reinterpret_cast<const char*>(base + (int64_t)row * row_stride) + c * 16;
-                    __builtin_amdgcn_global_load_lds(
-                        (const __attribute__((address_space(1))) void*)g,
-                        (__attribute__((address_space(3))) void*)(lds + slab * 1024), 16, 0, 0);
+                    async_load16(tile_base, goff[i], lds_base + slab * 1024);
                 } else {
                     *reinterpret_cast<i32x4*>(lds + slot * 16) = i32x4{0, 0, 0, 0};
                 }
@@ -259,18 +285,6 @@ constexpr int rowwise_pad() { return 16; }
 template <typename E, int D>
 constexpr int transposed_pad() {
     return Elem<E>::k16 ? (D * Elem<E>::kBytes >= 128 ? 64 : 0) : 32;
-}
-
-// One asynchronous 16-byte global->LDS copy per lane: lane l's data lands at lds_base + 16*l.
-// Written as inline asm so the compiler does not serialise later LDS reads behind it; the caller
-// orders things with wait_async_tiles() + a workgroup barrier.  lds_base must be wave-uniform.
-__device__ __forceinline__ void async_load16(const void* tile_base, int byte_off, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_base), "v"(byte_off), "s"(tile_base) : "memory");
-}
-
-__device__ __forceinline__ unsigned lds_address(const void* p) {
-    return (unsigned)(unsigned long long)(const __attribute__((address_space(3))) char*)p;
 }
 
 // Asynchronous staging of a ROWS x D tile into a PaddedTile.  Each wave instruction fills one
@@ -329,15 +343,16 @@ struct Resident {
     i32x4 c[NJ];
 };
 
-// Per-lane byte offsets of everything a wave reads from an LDS tile, computed once per kernel so
-// the inner loops issue LDS reads with no address arithmetic.  Offsets are for the first 32-row
-// block of a tile; block kb adds kb * BLOCK_BYTES (valid when LdsTile::kBlockAffine, otherwise the
-// address is recomputed).
+// Per-lane byte offsets of everything a wave reads from a swizzled LdsTile, computed once per
+// kernel; inside the loops an LDS address is "tile base + lane offset" plus an immediate.
+// Offsets are for the first 32-row block of a tile; block kb adds kb * BLOCK_BYTES (valid when
+// LdsTile::kBlockAffine, otherwise the address is recomputed).
 //   row[j]          16-byte chunk (row n, 2*j + h): the row-wise operand.  For 16-bit types one
 //                   MFMA operand (contraction slots 16*j + 8*h ..), for fp32 four (slots 8*j + 4*h ..).
 //   tr[db][s][w]    16-bit types: address this lane supplies to ds_read_b64_tr_b16 for the transposed
 //                   operand of head-dim block db, 16-row half s, first (w = 0) or second (w = 1)
-//                   group of four contraction rows.
+//                   group of four contraction rows.  When 16 rows are a whole number of swizzle
+//                   periods only s = 0 is stored and s = 1 is 16 rows further.
 // ds_read_b64_tr_b16 works on groups of 16 lanes: lane r of a group supplies the address of four
 // consecutive 16-bit elements X[k0 + r/4][n0 + 4*(r%4) ..] and lane i of the group receives
 // X[k0 + 0..3][n0 + i].
@@ -346,8 +361,11 @@ struct OperandOffsets {
     typedef LdsTile<E, D> L;
     static constexpr int NJ = L::CH / 2;
     static constexpr int DB = (D + 31) / 32;
+    static constexpr bool kHalfAffine = L::CH >= 16;  // +16 rows keeps the swizzle key (mod 16)
+    static constexpr int NS_TR = kHalfAffine ? 1 : 2;
+    static constexpr int ROW_BYTES = L::CH * 16;
     int row[NJ];
-    int tr[Elem<E>::k16 ? DB : 1][2][2];
+    int tr[Elem<E>::k16 ? DB : 1][NS_TR][2];
 
     __device__ __forceinline__ void init(int lane) {
         const int n = lane & 31, h = lane >> 5;
@@ -360,37 +378,38 @@ struct OperandOffsets {
                 int col = 32 * db + 16 * colgrp + 4 * (r & 3);
                 if (D < 32) col &= (D - 1);
 #pragma unroll
-                for (int s = 0; s < 2; s++)
+                for (int s = 0; s < NS_TR; s++)
 #pragma unroll
                     for (int w = 0; w < 2; w++) tr[db][s][w] = L::elem_off(16 * s + 8 * w + 4 * h + (r >> 2), col);
             }
         }
     }
 
-    __device__ __forceinline__ i32x4 row_chunk(const char* lds, int kb, int j, int lane) const {
+    __device__ __forceinline__ i32x4 row_chunk(const lds_char* tile, int kb, int j, int lane) const {
         if constexpr (L::kBlockAffine) {
-            return *reinterpret_cast<const i32x4*>(lds + row[j] + kb * L::BLOCK_BYTES);
+            return *reinterpret_cast<const lds_i32x4*>(tile + row[j] + kb * L::BLOCK_BYTES);
         } else {
-            return *reinterpret_cast<const i32x4*>(lds + L::chunk_off(32 * kb + (lane & 31), 2 * j + (lane >> 5)));
+            return *reinterpret_cast<const lds_i32x4*>(tile + L::chunk_off(32 * kb + (lane & 31), 2 * j + (lane >> 5)));
         }
     }
 
     // Transposed 16-bit operand: rows {32*kb + 16*s + 4*h + (0..3), + 8} at column 32*db + n.
-    __device__ __forceinline__ i32x4 tr_operand(const char* lds, int kb, int s, int db, int lane) const {
-        int o0, o1;
+    __device__ __forceinline__ i32x4 tr_operand(const lds_char* tile, int kb, int s, int db, int lane) const {
+        const lds_char *a0, *a1;
         if constexpr (L::kBlockAffine) {
-            o0 = tr[db][s][0] + kb * L::BLOCK_BYTES;
-            o1 = tr[db][s][1] + kb * L::BLOCK_BYTES;
+            const int imm = kb * L::BLOCK_BYTES + (kHalfAffine ? s * 16 * ROW_BYTES : 0);
+            a0 = tile + tr[db][kHalfAffine ? 0 : s][0] + imm;
+            a1 = tile + tr[db][kHalfAffine ? 0 : s][1] + imm;
         } else {
             const int r = lane & 15, colgrp = (lane >> 4) & 1, h = lane >> 5;
             int col = 32 * db + 16 * colgrp + 4 * (r & 3);
             if (D < 32) col &= (D - 1);
             const int rw = 32 * kb + 16 * s + 4 * h + (r >> 2);
-            o0 = L::elem_off(rw, col);
-            o1 = L::elem_off(rw + 8, col);
+            a0 = tile + L::elem_off(rw, col);
+            a1 = tile + L::elem_off(rw + 8, col);
         }
-        i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(lds + o0));
-        i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(lds + o1));
+        i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)a0);
+        i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)a1);
         i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         return __builtin_bit_cast(i32x4, v);
     }
@@ -398,40 +417,45 @@ struct OperandOffsets {
 
 // acc(32 rows of the LDS tile x 32 cols) += X[32*kb + 0..31][:] * B^T, B = resident rows.
 template <typename E, int D>
-__device__ __forceinline__ f32x16 mma_rowwise(const char* lds, int kb, const OperandOffsets<E, D>& ofs,
+__device__ __forceinline__ f32x16 mma_rowwise(const lds_char* tile, int kb, const OperandOffsets<E, D>& ofs,
                                               const Resident<E, D>& b, f32x16 acc, int lane) {
 #pragma unroll
-    for (int j = 0; j < Resident<E, D>::NJ; j++) acc = Elem<E>::mma(ofs.row_chunk(lds, kb, j, lane), b.c[j], acc);
+    for (int j = 0; j < Resident<E, D>::NJ; j++) acc = Elem<E>::mma(ofs.row_chunk(tile, kb, j, lane), b.c[j], acc);
     return acc;
 }
 
 // acc(32 out-rows x 32 cols) += X^T * P: contraction over the 32 rows of block kb of the LDS tile,
 // P a 32x32 accumulator-layout block (rows = contraction index) reused as B operand, output row
-// index = column 32*db + n of the LDS tile.
+// index = column 32*db + n of the LDS tile.  All DB head-dim blocks share the packed P operand.
 template <typename E, int D>
-__device__ __forceinline__ f32x16 mma_transposed(const char* lds, int kb, int db, const OperandOffsets<E, D>& ofs,
-                                                 f32x16 p, f32x16 acc, int lane) {
+__device__ __forceinline__ void mma_transposed(const lds_char* tile, int kb, const OperandOffsets<E, D>& ofs,
+                                               const f32x16& p, f32x16 (&acc)[(D + 31) / 32], int lane) {
+    constexpr int DB = (D + 31) / 32;
     if constexpr (Elem<E>::k16) {
 #pragma unroll
         for (int s = 0; s < 2; s++) {
             f32x8 ps;
 #pragma unroll
             for (int e = 0; e < 8; e++) ps[e] = p[8 * s + e];
-            acc = Elem<E>::mma(ofs.tr_operand(lds, kb, s, db, lane), Elem<E>::pack8(ps), acc);
+            const i32x4 bop = Elem<E>::pack8(ps);
+#pragma unroll
+            for (int db = 0; db < DB; db++) acc[db] = Elem<E>::mma(ofs.tr_operand(tile, kb, s, db, lane), bop, acc[db]);
         }
     } else {
         typedef LdsTile<E, D> L;
         int h = lane >> 5;
-        int col = 32 * db + (lane & 31);
-        if (D < 32) col &= (D - 1);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             int rw = 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
-            float a = *reinterpret_cast<const float*>(lds + L::elem_off(rw, col));
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, p[r], acc, 0, 0, 0);
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                int col = 32 * db + (lane & 31);
+                if (D < 32) col &= (D - 1);
+                float a = *reinterpret_cast<const lds_float*>(tile + L::elem_off(rw, col));
+                acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, p[r], acc[db], 0, 0, 0);
+            }
         }
     }
-    return acc;
 }
 
 // Load the resident operand chunks of the wave's 32 rows straight from global memory:

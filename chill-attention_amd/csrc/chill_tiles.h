@@ -37,12 +37,26 @@ constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
                       fwd_stages_for(streamed, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
 }
 
+// dQ LDS stage: swizzled (unpadded) K and V tiles; three stages when they fit in 144 KiB.
+constexpr int dq_stages_for(int streamed, int D, int dtype) {
+    return 3 * 2 * streamed * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
+}
+
 constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
-    const int waves = 4;
+    const int waves = fast16 ? 8 : 4;
     const int streamed = fast16 ? 64 : 32;
-    return TileConfig{waves * 32, streamed, waves, 2 * 2 * streamed * D * elem_bytes(dtype)};
+    return TileConfig{waves * 32, streamed, waves,
+                      dq_stages_for(streamed, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
+}
+
+// dK/dV LDS stage: swizzled Q and dO tiles plus the LSE2 and delta of their rows.
+constexpr int dkdv_stage_bytes(int streamed, int D, int dtype) {
+    return 2 * streamed * D * elem_bytes(dtype) + 2 * streamed * 4;
+}
+constexpr int dkdv_stages_for(int streamed, int D, int dtype) {
+    return 3 * dkdv_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
 
 constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
@@ -50,9 +64,8 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
     const int waves = 4;
     const int streamed = fast16 ? 64 : 32;
-    // double-buffered Q and dO tiles plus their LSE2 / delta vectors
     return TileConfig{waves * 32, streamed, waves,
-                      2 * (2 * streamed * D * elem_bytes(dtype) + 2 * streamed * 4)};
+                      dkdv_stages_for(streamed, D, dtype) * dkdv_stage_bytes(streamed, D, dtype)};
 }
 
 inline int tile_config(int mask_id, int D, int dtype, int pass, TileConfig* out) {
