@@ -279,12 +279,209 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
+// One workgroup owns TKR = 32 * NW / 2 key rows; their K and V tiles sit in LDS for the whole
+// kernel.  Streamed through the LDS ring: Q and dO tiles of 64 query rows with their LSE2 / delta,
+// for every query head of the GQA group in turn (chill_bwd_dkdv.py:156).
+//
+// Waves work in pairs on one 32-key block: wave w takes the first 32 query rows of every streamed
+// tile, wave w + NW/2 the second 32, each with its own dK^T / dV^T accumulators, which are summed
+// through LDS at the end.  Splitting the QUERY axis inside a pair keeps the per-wave state (two
+// 32 x D accumulators, no resident MFMA operands) within 256 registers, so two waves share a SIMD
+// and one wave's vector work hides behind the other's MFMAs, with no redundant MFMA work.
+template <typename E, int D, int MASK, int NW, int NS>
+__global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
+                                                       int wave_has_full_blocks) {
+    using ET = typename Elem<E>::type;
+    typedef LdsTile<E, D> L;
+    constexpr int NKB = NW / 2;      // 32-key blocks per workgroup
+    constexpr int TKR = NKB * 32;    // resident key rows per workgroup
+    constexpr int TQS = 64;          // streamed query rows per tile: 32 per wave of a pair
+    constexpr int NT = NW * 64;
+    constexpr int DB = (D + 31) / 32;
+    constexpr int NJ = L::CH / 2;
+    constexpr int KV_BYTES = L::bytes(TKR);
+    constexpr int TILE_BYTES = L::bytes(TQS);
+    constexpr int VEC_BYTES = TQS * 4;
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * VEC_BYTES;  // Q, dO, LSE2, delta
+    constexpr int RING_OFF = 2 * KV_BYTES;                        // K, V tiles first
+    static_assert(NS == 2, "two ring stages");
+    static_assert(DB * 16 * 256 * NKB <= RING_OFF + NS * STAGE_BYTES, "pair reduction reuses the LDS");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    if (item < 0) return;
+    const int bh = item / n_k_tiles;
+    // key tiles first-to-last: for causal-like masks the longest run first
+    const int ktile = item % n_k_tiles;
+    const int b = bh / p.H_kv;
+    const int hkv = bh % p.H_kv;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kblk = wave % NKB;   // which 32-key block
+    const int half = wave / NKB;   // which 32-row half of every streamed tile
+    const int n = lane & 31;
+    const int h = lane >> 5;
+
+    int seq_len = p.T;
+    if (p.lens != nullptr) seq_len = imin(p.lens[(int64_t)b * p.lens_stride], p.T);
+
+    const int kb0 = ktile * TKR;
+    ET* dkbase = reinterpret_cast<ET*>(p.dk) + b * p.sdk.b + hkv * p.sdk.h;
+    ET* dvbase = reinterpret_cast<ET*>(p.dv) + b * p.sdv.b + hkv * p.sdv.h;
+    if (kb0 >= seq_len) {
+        int nrows = imin(TKR, p.T - kb0);
+        zero_rows<E, D, NT>(dkbase, p.sdk.t, kb0, nrows, tid);
+        zero_rows<E, D, NT>(dvbase, p.sdv.t, kb0, nrows, tid);
+        return;
+    }
+
+    const TileRange wg = tile_range<MASK, false>(kb0, TKR, TQS, seq_len, false, p.margs);
+    const int n_tiles = wg.end - wg.start;
+    const int n_iters = n_tiles * p.group;
+
+    // resident K and V tiles
+    {
+        AsyncSwizzledLoader<E, D, TKR, NT> load_kv;
+        const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
+        const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
+        load_kv.init(p.sk.t, wave, lane);
+        load_kv.issue(kptr + (int64_t)kb0 * p.sk.t, p.T - kb0, smem, wave, lane);
+        load_kv.init(p.sv.t, wave, lane);
+        load_kv.issue(vptr + (int64_t)kb0 * p.sv.t, p.T - kb0, smem + KV_BYTES, wave, lane);
+    }
+
+    AsyncSwizzledLoader<E, D, TQS, NT> load_q, load_do;
+    load_q.init(p.sq.t, wave, lane);
+    load_do.init(p.sdo.t, wave, lane);
+    // iteration it = (group head g, q-tile)
+    auto issue_iter = [&](int it, int st_index) {
+        const int g = it / n_tiles;
+        const int q0 = (wg.start + it % n_tiles) * TQS;
+        const int hq = hkv * p.group + g;
+        char* st = smem + RING_OFF + st_index * STAGE_BYTES;
+        const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
+        const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
+        load_q.issue(qptr + (int64_t)q0 * p.sq.t, p.T - q0, st, wave, lane);
+        load_do.issue(doptr + (int64_t)q0 * p.sdo.t, p.T - q0, st + TILE_BYTES, wave, lane);
+        if (wave == NW - 1) {
+            // LSE2 and delta of the tile's rows; rows past the end of the tensor read as zero
+            const float* lse = p.lse + b * p.lse_b + hq * p.lse_h + q0;
+            const float* del = p.delta + b * p.delta_b + hq * p.delta_h + q0;
+            char* vec = st + 2 * TILE_BYTES;
+            if (q0 + lane < p.T) {
+                async_load4(lse, lane * 4, lds_address(vec));
+                async_load4(del, lane * 4, lds_address(vec + VEC_BYTES));
+            } else {
+                reinterpret_cast<float*>(vec)[lane] = 0.f;
+                reinterpret_cast<float*>(vec + VEC_BYTES)[lane] = 0.f;
+            }
+        }
+    };
+    if (n_iters > 0) issue_iter(0, 0);
+
+    const int kw = kb0 + 32 * kblk;
+    const int k_pos = kw + n;
+    OperandOffsets<E, D> ofs;
+    ofs.init(lane);
+
+    TileRange wr = {wg.start, wg.start, wg.start, wg.start};
+    if (kw < seq_len) wr = tile_range<MASK, false>(kw, 32, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
+    const int ta = wr.start - wg.start, tb = wr.end - wg.start;
+    const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
+
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int i = 0; i < DB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            dk[i][r] = 0.f;
+            dv[i][r] = 0.f;
+        }
+    const float scale = p.scale_log2;
+    const lds_char* lds0 = (const lds_char*)smem;
+    const lds_char* k_tile = lds0;
+    const lds_char* v_tile = lds0 + KV_BYTES;
+
+    int st_cur = NS - 1;
+    int tile = -1;  // position of iteration `it` inside the q-tile range (it % n_tiles)
+    for (int it = 0; it < n_iters; it++) {
+        wait_async_tiles();
+        __syncthreads();
+        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+        tile = tile + 1 == n_tiles ? 0 : tile + 1;
+        if (it + 1 < n_iters) issue_iter(it + 1, st_cur + 1 == NS ? 0 : st_cur + 1);
+        if (tile < ta || tile >= tb) continue;
+        const lds_char* q_tile = lds0 + RING_OFF + st_cur * STAGE_BYTES;
+        const lds_char* do_tile = q_tile + TILE_BYTES;
+        const lds_float* vec = reinterpret_cast<const lds_float*>(q_tile + 2 * TILE_BYTES) + 32 * half;
+        const bool full = (tile >= fa) && (tile < fb);
+        const int q0 = (wg.start + tile) * TQS + 32 * half;
+
+        // S = Q K^T, dP = dO V^T: both operands from LDS
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            s[r] = 0.f;
+            dp[r] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
+            dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
+        }
+        f32x4 lse4[4], del4[4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+            lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
+            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
+        }
+        auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
+            q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
+            k = k_pos;
+            lse = lse4[r / 4][r % 4];
+            delta = del4[r / 4][r % 4];
+        };
+        if (full)
+            softmax_grad_block<MASK, false>(s, dp, scale, seq_len, p.margs, pos);
+        else
+            softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
+        mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);  // dV^T += dO^T P
+        mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);  // dK^T += Q^T dS
+    }
+
+    // sum the two waves of a pair through LDS (one accumulator at a time), then store
+    float* red = reinterpret_cast<float*>(smem) + kblk * (DB * 16 * 64) + lane;
+    auto reduce_and_store = [&](f32x16 (&acc)[DB], ET* base, int64_t row_stride, float mult) {
+        __syncthreads();  // everyone is done with the tiles (or with the previous round)
+        if (half == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) red[(db * 16 + r) * 64] = acc[db][r];
+        }
+        __syncthreads();
+        if (half == 0) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[db][r] += red[(db * 16 + r) * 64];
+            if (k_pos < p.T) store_row_transposed<E, D>(base + (int64_t)k_pos * row_stride, acc, mult, k_pos < seq_len, h);
+        }
+    };
+    reduce_and_store(dk, dkbase, p.sdk.t, p.sm_scale);
+    reduce_and_store(dv, dvbase, p.sdv.t, 1.f);
+}
+
+// ------------------------------------------------------------------------------------------ dK, dV (wide rows)
+// Variant for rows too long for the paired kernel's LDS budget (more than 256 bytes per row):
 // Resident: 32 key rows per wave (K, V as B operands).  Streamed through the LDS ring: Q and dO
 // tiles of TQS query rows with their LSE2 / delta, for every query head of the GQA group in turn
 // (chill_bwd_dkdv.py:156).  Steps of 32 queries; S and dP of step t+1 are issued before the vector
 // work of step t.
 template <typename E, int D, int MASK, int NW, int TQS, int NS>
-__global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
+__global__ __launch_bounds__(NW * 64) void dkdv_wide_kernel(BwdParams p, int n_k_tiles, int total_items,
                                                        int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     constexpr int TKR = NW * 32;  // resident key rows per workgroup
@@ -475,19 +672,26 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
 
 template <typename E, int D>
 int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
-    const int64_t max_stride = p.sq.t > p.sdo.t ? p.sq.t : p.sdo.t;
+    int64_t max_stride = p.sq.t > p.sdo.t ? p.sq.t : p.sdo.t;
+    if (p.sk.t > max_stride) max_stride = p.sk.t;
+    if (p.sv.t > max_stride) max_stride = p.sv.t;
     if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType);
-        static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
-        constexpr int NS = dkdv_stages_for(cfg.streamed, D, Elem<E>::kDType);
+        constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType);
+        static_assert(paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64) : (cfg.rows == cfg.waves * 32),
+                      "tile table and kernel shape disagree");
         const int n_k_tiles = cdiv(p.T, cfg.rows);
         const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        auto kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
+        void (*kern)(BwdParams, int, int, int);
+        if constexpr (paired)
+            kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, 2>;
+        else
+            kern = dkdv_wide_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, dkdv_wide_stages(cfg.streamed, D, Elem<E>::kDType)>;
         // mask rule order is (q tile, k tile): the streamed tile is the q tile here
         const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, 32, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {

@@ -51,21 +51,25 @@ constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
                       dq_stages_for(streamed, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
 }
 
-// dK/dV LDS stage: swizzled Q and dO tiles plus the LSE2 and delta of their rows.
-constexpr int dkdv_stage_bytes(int streamed, int D, int dtype) {
+// dK/dV, rows of at most 256 bytes ("paired" kernel): a workgroup of 8 waves owns 128 key rows;
+// pairs of waves share a 32-key block and split the streamed 64-row query tiles.  LDS: the resident
+// K and V tiles plus two ring stages of swizzled Q and dO tiles with the LSE2 and delta of their rows.
+// Longer rows ("wide" kernel): 4 waves own 128 key rows with K, V resident in registers; the ring
+// holds 32-row Q and dO tiles.
+constexpr bool dkdv_is_paired(int D, int dtype) { return D * elem_bytes(dtype) <= 256; }
+constexpr int dkdv_wide_stage_bytes(int streamed, int D, int dtype) {
     return 2 * streamed * D * elem_bytes(dtype) + 2 * streamed * 4;
 }
-constexpr int dkdv_stages_for(int streamed, int D, int dtype) {
-    return 3 * dkdv_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
+constexpr int dkdv_wide_stages(int streamed, int D, int dtype) {
+    return 3 * dkdv_wide_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
 
 constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
-    const bool fast16 = dtype != CHILL_F32 && D <= 128;
-    const int waves = 4;
-    const int streamed = fast16 ? 64 : 32;
-    return TileConfig{waves * 32, streamed, waves,
-                      dkdv_stages_for(streamed, D, dtype) * dkdv_stage_bytes(streamed, D, dtype)};
+    const int row_bytes = D * elem_bytes(dtype);
+    if (dkdv_is_paired(D, dtype))
+        return TileConfig{128, 64, 8, 2 * 128 * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4)};
+    return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
 }
 
 inline int tile_config(int mask_id, int D, int dtype, int pass, TileConfig* out) {
