@@ -196,7 +196,6 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
         dpdst = mma_rowwise<E, D>(stage + TILE_BYTES, kb, ofs, dof, dpdst, lane);
     };
 
-    f32x16 s[2], dp[2];
     const lds_char* lds0 = (const lds_char*)smem;
     // the resident operands must have arrived before the loop, where the only vector-memory traffic
     // is the async tile loads and no compiler-placed wait may cover them
@@ -214,20 +213,12 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
         if (i + LA + 1 < n_tiles) issue_tile(i + LA + 1, st_issue);
         if (i < ta || i >= tb) continue;
         const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
-        const lds_char* stage_next = lds0 + (st_cur + 1 == NS ? 0 : st_cur + 1) * STAGE_BYTES;
         const bool full = (i >= fa) && (i < fb);
         const int k0 = (wg.start + i) * TK;
-        if (LA == 0 || i == ta) gemms(s[0], dp[0], stage, 0);
-
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
-            f32x16& cs = s[kb & 1];
-            f32x16& cdp = dp[kb & 1];
-            if (kb + 1 < KB) {
-                gemms(s[(kb + 1) & 1], dp[(kb + 1) & 1], stage, kb + 1);
-            } else if (LA >= 1 && i + 1 < tb) {
-                gemms(s[(kb + 1) & 1], dp[(kb + 1) & 1], stage_next, 0);
-            }
+            f32x16 cs, cdp;
+            gemms(cs, cdp, stage, kb);
             auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
                 q = q_pos;
                 k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
@@ -240,10 +231,6 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
                 softmax_grad_block<MASK, true>(cs, cdp, scale, seq_len, p.margs, pos);
             // dQ^T += K^T dS^T
             mma_transposed<E, D>(stage, kb, ofs, cdp, dq, lane);
-        }
-        if (KB & 1) {
-            s[0] = s[1];
-            dp[0] = dp[1];
         }
     }
 
