@@ -108,10 +108,11 @@ def test_tile_table():
             for D in (16, 32, 64, 128, 256):
                 for p in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKDV):
                     c = tile_config(mask, D, dt, p)
-                    assert c["rows"] == 32 * c["waves"] and c["streamed"] % 32 == 0
+                    # one wave per 32 resident rows, or (dK/dV) a pair of waves per 32 rows
+                    assert c["rows"] in (32 * c["waves"], 16 * c["waves"]) and c["streamed"] % 32 == 0
                     assert 0 < c["lds_bytes"] <= 160 * 1024
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
-    assert tq == 32 * waves
+    assert tq == 32 * waves and tk % 32 == 0
     (dq_q, dq_k, _), (dk_q, dk_k, _) = _get_default_config_bwd(128, torch.bfloat16)
     assert dq_q % 32 == 0 and dk_k % 32 == 0
     out = (ctypes.c_int32 * 4)()
