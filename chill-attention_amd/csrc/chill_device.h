@@ -239,13 +239,18 @@ struct AsyncSwizzledLoader {
     __device__ __forceinline__ void issue(const typename Elem<E>::type* tile_base, int rows_valid, char* lds,
                                           int wave, int lane) const {
         const unsigned lds_base = lds_address(lds);
+        if (rows_valid >= ROWS) {
 #pragma unroll
-        for (int i = 0; i < PER_WAVE; i++) {
-            const int slab = i * NWV + wave;
-            if (SLABS % NWV != 0 && slab >= SLABS) continue;
-            if (rows_valid >= ROWS) {
+            for (int i = 0; i < PER_WAVE; i++) {
+                const int slab = i * NWV + wave;
+                if (SLABS % NWV != 0 && slab >= SLABS) continue;
                 async_load16(tile_base, goff[i], lds_base + slab * 1024);
-            } else {
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < PER_WAVE; i++) {
+                const int slab = i * NWV + wave;
+                if (SLABS % NWV != 0 && slab >= SLABS) continue;
                 int slot = slab * 64 + lane;
                 int row = L::phys(slot) / L::CH;
                 if (row < rows_valid) {
@@ -288,7 +293,7 @@ constexpr int transposed_pad() {
 }
 
 // Asynchronous staging of a ROWS x D tile into a PaddedTile.  Each wave instruction fills one
-// 1 KiB slab; a lane's slot maps to (row, chunk) = (slot / CHP, slot % CHP), pad slots are skipped.
+// 1 KiB slab; a lane's slot maps to (row, chunk) = (slot / CHP, slot % CHP).
 // The per-lane global offsets are computed once (init) because the tile geometry never changes.
 template <typename E, int D, int PAD, int ROWS, int NT>
 struct AsyncPaddedLoader {
@@ -297,14 +302,17 @@ struct AsyncPaddedLoader {
     static constexpr int SLABS = (SLOTS + 63) / 64;
     static constexpr int NWV = NT / 64;
     static constexpr int PER_WAVE = (SLABS + NWV - 1) / NWV;
-    int goff[PER_WAVE];  // byte offset from the tile's first row, -1 for a pad / unused slot
+    static constexpr bool kPartialLastSlab = SLOTS % 64 != 0;
+    // byte offset from the tile's first row.  Pad slots fetch (harmlessly) the first chunk of
+    // their row, so a full tile needs no lane masking; -1 marks slots past the end of the tile.
+    int goff[PER_WAVE];
 
     __device__ __forceinline__ void init(int64_t row_stride, int wave, int lane) {
 #pragma unroll
         for (int i = 0; i < PER_WAVE; i++) {
             int slot = (i * NWV + wave) * 64 + lane;
             int row = slot / P::CHP, c = slot % P::CHP;
-            goff[i] = (slot < SLOTS && c < P::CH) ? (int)(row * row_stride * Elem<E>::kBytes) + c * 16 : -1;
+            goff[i] = slot < SLOTS ? (int)(row * row_stride * Elem<E>::kBytes) + (c < P::CH ? c * 16 : 0) : -1;
         }
     }
 
@@ -312,14 +320,23 @@ struct AsyncPaddedLoader {
     __device__ __forceinline__ void issue(const typename Elem<E>::type* tile_base, int64_t row_stride,
                                           int rows_valid, char* lds, int wave, int lane) const {
         const unsigned lds_base = lds_address(lds);
+        if (rows_valid >= ROWS) {
 #pragma unroll
-        for (int i = 0; i < PER_WAVE; i++) {
-            const int slab = i * NWV + wave;
-            if (SLABS % NWV != 0 && slab >= SLABS) continue;
-            if (rows_valid >= ROWS) {
-                if (goff[i] >= 0) async_load16(tile_base, goff[i], lds_base + slab * 1024);
-            } else {
-                // ragged last tile: rows past the end of the tensor read as zeros
+            for (int i = 0; i < PER_WAVE; i++) {
+                const int slab = i * NWV + wave;
+                if (SLABS % NWV != 0 && slab >= SLABS) continue;
+                if (kPartialLastSlab && (i + 1) * NWV >= SLABS) {
+                    if (goff[i] >= 0) async_load16(tile_base, goff[i], lds_base + slab * 1024);
+                } else {
+                    async_load16(tile_base, goff[i], lds_base + slab * 1024);
+                }
+            }
+        } else {
+            // ragged last tile: rows past the end of the tensor read as zeros
+#pragma unroll
+            for (int i = 0; i < PER_WAVE; i++) {
+                const int slab = i * NWV + wave;
+                if (SLABS % NWV != 0 && slab >= SLABS) continue;
                 int slot = slab * 64 + lane;
                 int row = slot / P::CHP, c = slot % P::CHP;
                 if (slot < SLOTS && c < P::CH) {

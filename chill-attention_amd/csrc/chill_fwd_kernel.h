@@ -40,9 +40,10 @@ struct FwdLds {
     static constexpr int STAGE_BYTES = K_BYTES + V_BYTES;
 };
 
+// One q-tile (TQ = 32 * NW query rows of one head) from start to finish.
 template <typename E, int D, int MASK, int NW, int TK, int NS>
-__global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
-                                                      int wave_has_full_blocks) {
+__device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b, int hd, int qt,
+                                           int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     using M = Mask<MASK>;
     typedef FwdLds<E, D, TK> Lds;
@@ -55,15 +56,6 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
     constexpr int NJ = KT::CH / 2;      // 16-byte chunk pairs along the head dim
     constexpr int LA = NS - 2;          // tiles certified resident ahead of the one being consumed
     static_assert(NS == 2 || NS == 3, "two or three LDS stages");
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-
-    const int item = xcd_contiguous_item(blockIdx.x, total_items);
-    if (item < 0) return;
-    const int bh = item / n_q_tiles;
-    // q-tiles of one head are issued last-first: for causal-like masks the longest run first
-    const int qt = n_q_tiles - 1 - item % n_q_tiles;
-    const int b = bh / p.H;
-    const int hd = bh % p.H;
     const int hkv = hd / p.group;
 
     const int tid = threadIdx.x;
@@ -142,14 +134,22 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
     const bool negate = p.scale_log2 < 0.f;  // max(scale * s) = |scale| * max(sign * s)
     const float scale = negate ? -p.scale_log2 : p.scale_log2;
 
-    // S^T block of step kb of the tile at LDS address `stage`:  K[32*kb + 0..31][:] Q^T
-    auto scores = [&](f32x16& dst, const lds_char* stage, int kb) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) dst[r] = 0.f;
+    // K operands of the score block of step kb of the tile at `stage` (rows 32*kb .. 32*kb+31),
+    // read one step ahead of the MFMAs that consume them
+    struct KOperands {
+        i32x4 c[NJ];
+    };
+    auto load_k_operands = [&](KOperands& ko, const lds_char* stage, int kb) {
         const lds_char* base = stage + k_lane + kb * 32 * KT::PITCH;
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
-            dst = Elem<E>::mma(*reinterpret_cast<const lds_i32x4*>(base + j * 32), qf.c[j], dst);
+        for (int j = 0; j < NJ; j++) ko.c[j] = *reinterpret_cast<const lds_i32x4*>(base + j * 32);
+    };
+    // S^T block: K[32 rows][:] Q^T
+    auto scores = [&](f32x16& dst, const KOperands& ko) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) dst[r] = 0.f;
+#pragma unroll
+        for (int j = 0; j < NJ; j++) dst = Elem<E>::mma(ko.c[j], qf.c[j], dst);
     };
     // sign, mask and block max (scaled) of a score block
     auto prepare = [&](f32x16& sc, bool full, int key0) -> float {
@@ -170,9 +170,28 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
         for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
         return max_across_halves(mx) * scale;
     };
-    // O^T += V^T P^T for step kb of the tile at `stage`
-    auto accumulate = [&](const f32x16& pr, const lds_char* stage, int kb) {
-        const lds_char* base = stage + v_lane + kb * 32 * VT::PITCH;
+    // A operands of O^T += V^T P^T for step kb of the tile at `stage`: V^T blocks, read up front so
+    // that their LDS latency hides behind the score MFMAs and the softmax of the step.
+    // 16-bit: vt[s2][db] = transposed operand of keys 16*s2 .. 16*s2+15; fp32: read at use.
+    struct VOperands {
+        i16x4 lo[Elem<E>::k16 ? 2 : 1][Elem<E>::k16 ? DB : 1];
+        i16x4 hi[Elem<E>::k16 ? 2 : 1][Elem<E>::k16 ? DB : 1];
+    };
+    auto load_v_operands = [&](VOperands& vo, const lds_char* stage, int kb) {
+        if constexpr (Elem<E>::k16) {
+            const lds_char* base = stage + v_lane + kb * 32 * VT::PITCH;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    const lds_char* a0 = base + (16 * s2) * VT::PITCH + db * 64;
+                    vo.lo[s2][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)a0);
+                    vo.hi[s2][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(a0 + 8 * VT::PITCH));
+                }
+        }
+    };
+    // O^T += V^T P^T
+    auto accumulate = [&](const f32x16& pr, const VOperands& vo, const lds_char* stage, int kb) {
         if constexpr (Elem<E>::k16) {
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
@@ -182,14 +201,12 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
                 const i32x4 bop = Elem<E>::pack8(ps);
 #pragma unroll
                 for (int db = 0; db < DB; db++) {
-                    const lds_char* a0 = base + (16 * s2) * VT::PITCH + db * 64;
-                    i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)a0);
-                    i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(a0 + 8 * VT::PITCH));
-                    i16x8 av = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    i16x8 av = __builtin_shufflevector(vo.lo[s2][db], vo.hi[s2][db], 0, 1, 2, 3, 4, 5, 6, 7);
                     o[db] = Elem<E>::mma(__builtin_bit_cast(i32x4, av), bop, o[db]);
                 }
             }
         } else {
+            const lds_char* base = stage + v_lane + kb * 32 * VT::PITCH;
 #pragma unroll
             for (int r = 0; r < 16; r++)
 #pragma unroll
@@ -201,6 +218,7 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
     };
 
     f32x16 s[2];         // scores of the current and of the next step
+    KOperands ka;        // K operands of the next score block
     float mx_cur = 0.f;  // block max of s[current], already scaled
     const lds_char* lds0 = (const lds_char*)smem;
     // Q must have arrived before the loop: inside it the only vector-memory traffic is the async
@@ -224,8 +242,11 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
         const bool full_next = (i + 1 >= fa) && (i + 1 < fb);
         const int k0 = (wg.start + i) * TK;
         if (LA == 0 || i == ta) {
-            scores(s[0], stage, 0);
+            load_k_operands(ka, stage, 0);
+            scores(s[0], ka);
             mx_cur = prepare(s[0], full, k0);
+            // operands of the step after (with one step per tile they are read at the top of the step)
+            if (KB > 1) load_k_operands(ka, stage, 1);
         }
 
 #pragma unroll
@@ -246,14 +267,15 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
 #pragma unroll
                     for (int r = 0; r < 16; r++) o[db][r] *= alpha;
             }
-            // scores of the next step fly while this step's softmax runs
+            if (KB == 1 && LA >= 1 && i + 1 < tb) load_k_operands(ka, stage_next, 0);
+            // V operands of this step: issued now, consumed after the softmax
+            VOperands vo;
+            load_v_operands(vo, stage, kb);
+            __builtin_amdgcn_sched_barrier(0);
+            // scores of the next step (operands already in registers) fly while this step's softmax runs
             const bool in_tile = kb + 1 < KB;
             const bool have_next = in_tile || (LA >= 1 && i + 1 < tb);
-            if (in_tile) {
-                scores(nxt, stage, kb + 1);
-            } else if (LA >= 1 && i + 1 < tb) {
-                scores(nxt, stage_next, 0);
-            }
+            if (have_next) scores(nxt, ka);
             float psum = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
@@ -262,7 +284,14 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
                 psum += pv;
             }
             l_run += psum;
-            accumulate(cur, stage, kb);
+            __builtin_amdgcn_sched_barrier(0);
+            // K operands of the step after next, behind the score MFMAs that read the old ones
+            if (kb + 2 < KB) {
+                load_k_operands(ka, stage, kb + 2);
+            } else if (KB > 1 && LA >= 1 && i + 1 < tb) {
+                load_k_operands(ka, stage_next, kb + 2 - KB);
+            }
+            accumulate(cur, vo, stage, kb);
             if (have_next) mx_cur = in_tile ? prepare(nxt, full, k0 + 32 * (kb + 1)) : prepare(nxt, full_next, k0 + TK);
         }
         if (KB & 1) s[0] = s[1];  // odd step count: the prefetched scores sit in the other buffer
@@ -281,6 +310,28 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
     }
 }
 
+// One workgroup per (batch, head, PAIR of q-tiles): tile j from the end, then tile j from the
+// start.  For causal-like masks the work of a q-tile grows with its index, so the two halves of a
+// pair add up to the same amount for every workgroup and the grid finishes without a tail.
+template <typename E, int D, int MASK, int NW, int TK, int NS>
+__global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
+                                                      int wave_has_full_blocks) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    if (item < 0) return;
+    const int n_pairs = (n_q_tiles + 1) / 2;
+    const int bh = item / n_pairs;
+    const int j = item % n_pairs;
+    const int b = bh / p.H;
+    const int hd = bh % p.H;
+    const int qt_hi = n_q_tiles - 1 - j;
+    fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, wave_has_full_blocks);
+    if (j != qt_hi) {
+        __syncthreads();  // the LDS ring is reused
+        fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
+    }
+}
+
 // Launcher for one (element type, head dim); dispatches on the mask id and takes the tile shape
 // from the static table.
 template <typename E, int D>
@@ -296,7 +347,7 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES,
                       "table and kernel disagree on LDS");
         const int n_q_tiles = cdiv(p.T, cfg.rows);
-        const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
+        const int64_t total64 = (int64_t)p.B * p.H * ((n_q_tiles + 1) / 2);
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
