@@ -32,6 +32,16 @@ sys.path.insert(0, os.path.join(ROOT, "chill-attention_amd"))
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}  # MI355X dense MFMA
 PEAK_HBM_GBS = 8000.0
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), scaled by what
+# the same counters read for a plain 1 GiB copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
+# the summaries of those runs are kept under profiles/.  (workload, kernel) -> bytes
+MEASURED_TRAFFIC = {
+    ("C3", "chill_fwd"): (657300 * 2.0 + 266200) * 1024,
+    ("C3", "chill_bwd_delta"): (262200 * 2.0 + 4115) * 1024,
+    ("C3", "chill_bwd_dkdv"): (528500 * 2.0 + 524300) * 1024,
+    ("C3", "chill_bwd_dq"): (735100 * 2.0 + 262100) * 1024,
+}
+
 # name -> (mask ctor name, args, dtype, B, H, T, D, seed, sigma)
 WORKLOADS = {
     "C1": ("CausalChillMask", (), "f32", 1, 2, 256, 64, 0, 1.0),
@@ -158,6 +168,10 @@ def main():
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--mode", default="fwd+bwd", choices=["fwd", "fwd+bwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch one plain 1 GiB device copy (1 GiB read + 1 GiB written) before the warm-up: "
+                         "the known-size dispatch that scales the FETCH_SIZE / WRITE_SIZE counters of a "
+                         "rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE MI355X; every box has one GPU and the hot path "
@@ -178,6 +192,14 @@ def main():
     q, k, v, do = make_inputs(torch, B, H, T, D, dtype, seed, sigma, dev)
     run = Runner(torch, ca, mask, q, k, v, do, D ** -0.5)
     kernels = run.kernels(mode)
+
+    if args.copy_probe:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         for _, fn in kernels:
@@ -222,7 +244,14 @@ def main():
         roof = {"kernel": dom_name, "bound": "mfma", "achieved": alg / (k_ms[dom] * 1e-3) / 1e12, "peak": peak,
                 "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, dom_name))
+    roof["traffic_unit"] = "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-scaled)"
+    roof["algorithmic_bytes"] = {
+        "chill_fwd": 4.0 * B * H * T * D * es + 4.0 * B * H * T,
+        "chill_bwd_delta": 2.0 * B * H * T * D * es + 4.0 * B * H * T,
+        "chill_bwd_dkdv": 6.0 * B * H * T * D * es + 8.0 * B * H * T,
+        "chill_bwd_dq": 5.0 * B * H * T * D * es + 8.0 * B * H * T,
+    }[dom_name]
     roof["avg_launch_ms"] = k_ms[dom]
 
     out = {

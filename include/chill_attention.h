@@ -87,8 +87,9 @@ typedef enum ChillPass {
 
 /* Forward: O = softmax(mask(Q K^T * sm_scale)) V, optional LSE2.
  * Replaces the launch of _chill_attn_fwd (chill_fwd.py:21-359) at chill.py:207, grid chill.py:122-123.
- * `o` must be zero-initialised by the caller when lens != NULL (rows of q-tiles lying entirely
- * at or beyond lens[b] are not written, chill_fwd.py:70-71; the adapter zero-fills at chill.py:96).
+ * Every row of `o` (and of `lse`) is written: rows at or beyond lens[b] and rows whose q-tile has
+ * no k-tile receive 0 (the reference leaves them at the adapter's zero-fill, chill.py:96 and
+ * chill_fwd.py:70-71), so the caller may pass uninitialised memory.
  * `lse` may be NULL (return_lse = False). */
 int chill_fwd(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
               const ChillTensor4* o,
@@ -106,8 +107,8 @@ int chill_bwd_delta(const ChillTensor4* o, const ChillTensor4* d_o,
                     int32_t dtype, void* stream);
 
 /* dQ: replaces the dq branch of _chill_attn_bwd (chill_bwd.py:93-129 ->
- * chill_bwd_dq.py:15-397), launched at chill.py:442.  `dq` is written for every row < seq_len of
- * q-tiles that start below seq_len; the caller zero-fills it when lens != NULL (chill.py:292). */
+ * chill_bwd_dq.py:15-397), launched at chill.py:442.  Every row of `dq` is written; rows at or
+ * beyond lens[b] receive 0 (the reference relies on the adapter's zero-fill, chill.py:292). */
 int chill_bwd_dq(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
                  const ChillTensor4* d_o, const ChillTensor4* dq,
                  const float* lse, const int64_t lse_stride[3],
@@ -119,8 +120,9 @@ int chill_bwd_dq(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor
 
 /* dK, dV: replaces the dkdv branch of _chill_attn_bwd (chill_bwd.py:130-167 ->
  * chill_bwd_dkdv.py:15-509), launched at chill.py:442.  One workgroup per (batch, kv head,
- * k-tile); the GQA group loop (chill_bwd_dkdv.py:156) runs inside it.  The caller zero-fills
- * dk / dv when lens != NULL (chill.py:293-294). */
+ * k-tile); the GQA group loop (chill_bwd_dkdv.py:156) runs inside it.  Every row of `dk` and `dv`
+ * is written; rows at or beyond lens[b] receive 0 (the reference relies on the adapter's
+ * zero-fill, chill.py:293-294). */
 int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
                    const ChillTensor4* d_o, const ChillTensor4* dk, const ChillTensor4* dv,
                    const float* lse, const int64_t lse_stride[3],
