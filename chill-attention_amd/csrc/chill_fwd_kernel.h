@@ -22,6 +22,8 @@
 // inside its own full range.  The workgroup stages the hull of its waves' ranges.
 #pragma once
 
+#include <type_traits>
+
 #include "chill_device.h"
 #include "chill_params.h"
 #include "chill_tiles.h"
@@ -30,6 +32,9 @@ namespace chill {
 
 // Lazy-rescale threshold of the online softmax, in log2 units: P stays below 2^kRescaleTau.
 constexpr float kRescaleTau = 8.0f;
+#ifndef CHILL_SCHED_GROUPS
+#define CHILL_SCHED_GROUPS 1
+#endif
 
 template <typename E, int D, int TK>
 struct FwdLds {
@@ -131,8 +136,9 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
     float m_use = 0.f;        // m_run, or 0 while the row has seen no unmasked key
     float l_run = 0.f;        // this lane's share of the row sum
     const int q_pos = qw + n;
-    const bool negate = p.scale_log2 < 0.f;  // max(scale * s) = |scale| * max(sign * s)
-    const float scale = negate ? -p.scale_log2 : p.scale_log2;
+    // A negative scale reverses the order of the scores: the sign goes into Q, the softmax works
+    // with |scale| (max(scale * s) = |scale| * max(sign * s)).
+    const float scale = fabsf(p.scale_log2);
 
     // K operands of the score block of step kb of the tile at `stage` (rows 32*kb .. 32*kb+31),
     // read one step ahead of the MFMAs that consume them
@@ -151,12 +157,8 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
 #pragma unroll
         for (int j = 0; j < NJ; j++) dst = Elem<E>::mma(ko.c[j], qf.c[j], dst);
     };
-    // sign, mask and block max (scaled) of a score block
+    // mask and block max (scaled) of a score block
     auto prepare = [&](f32x16& sc, bool full, int key0) -> float {
-        if (negate) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) sc[r] = -sc[r];
-        }
         if (!full) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
@@ -224,7 +226,73 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
     // Q must have arrived before the loop: inside it the only vector-memory traffic is the async
     // tile loads, and the compiler must not place a wait for them in front of the first MFMA
 #pragma unroll
-    for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(qf.c[j]));
+    for (int j = 0; j < NJ; j++) {
+        if (p.scale_log2 < 0.f) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) qf.c[j][e] ^= Elem<E>::k16 ? (int)0x80008000 : (int)0x80000000;
+        }
+        asm volatile("" ::"v"(qf.c[j]));
+    }
+
+    // One step: softmax of the current 32-key block and its share of O, with the scores of the next
+    // block issued first.  With a tile resident ahead (LA >= 1) the step reads the next block
+    // unconditionally — a wave's last step reads a stage whose contents it never uses — so that
+    // between the rare rescale branch and the mask branch the step is one basic block in which
+    // the instruction groups below interleave matrix and vector work.
+    auto step = [&](const lds_char* stage, const lds_char* stage_next, int kb, bool full, bool full_next, int k0) {
+        f32x16& cur = s[kb & 1];
+        f32x16& nxt = s[(kb + 1) & 1];
+        // rare path: raise the reference max and rescale what has been accumulated
+        const bool raise = mx_cur > m_run + kRescaleTau;
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+            const float m_new = raise ? mx_cur : m_run;
+            const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = fast_exp2(m_use - m_use_new);
+            m_run = m_new;
+            m_use = m_use_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        }
+        const bool in_tile = kb + 1 < KB;
+        const bool have_next = in_tile || LA >= 1;
+        if (KB == 1 && LA >= 1) load_k_operands(ka, stage_next, 0);
+        // V operands of this step: issued now, consumed after the softmax
+        VOperands vo;
+        load_v_operands(vo, stage, kb);
+        __builtin_amdgcn_sched_barrier(0);
+        // scores of the next step (operands already in registers) fly while this step's softmax runs
+        if (have_next) scores(nxt, ka);
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float pv = fast_exp2(__builtin_fmaf(cur[r], scale, -m_use));
+            cur[r] = pv;
+            psum += pv;
+        }
+        l_run += psum;
+        if constexpr (Elem<E>::k16 && CHILL_SCHED_GROUPS) {
+            // every score MFMA is followed by its share of the softmax
+            if (have_next) {
+#pragma unroll
+                for (int j = 0; j < NJ; j++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x402, (48 + NJ - 1) / NJ, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // K operands of the step after next, behind the score MFMAs that read the old ones
+        if (kb + 2 < KB) {
+            load_k_operands(ka, stage, kb + 2);
+        } else if (KB > 1 && LA >= 1) {
+            load_k_operands(ka, stage_next, kb + 2 - KB);
+        }
+        accumulate(cur, vo, stage, kb);
+        if (have_next) mx_cur = in_tile ? prepare(nxt, full, k0 + 32 * (kb + 1)) : prepare(nxt, full_next, k0 + TK);
+    };
 
     int st_cur = NS - 1;  // LDS stage of tile i (advanced at the top of the loop)
     int st_issue = LA;    // LDS stage the next issued tile goes to
@@ -248,52 +316,8 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
             // operands of the step after (with one step per tile they are read at the top of the step)
             if (KB > 1) load_k_operands(ka, stage, 1);
         }
-
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++) {
-            f32x16& cur = s[kb & 1];
-            f32x16& nxt = s[(kb + 1) & 1];
-            // rare path: raise the reference max and rescale what has been accumulated
-            const bool raise = mx_cur > m_run + kRescaleTau;
-            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-                const float m_new = raise ? mx_cur : m_run;
-                const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
-                const float alpha = fast_exp2(m_use - m_use_new);
-                m_run = m_new;
-                m_use = m_use_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int db = 0; db < DB; db++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) o[db][r] *= alpha;
-            }
-            if (KB == 1 && LA >= 1 && i + 1 < tb) load_k_operands(ka, stage_next, 0);
-            // V operands of this step: issued now, consumed after the softmax
-            VOperands vo;
-            load_v_operands(vo, stage, kb);
-            __builtin_amdgcn_sched_barrier(0);
-            // scores of the next step (operands already in registers) fly while this step's softmax runs
-            const bool in_tile = kb + 1 < KB;
-            const bool have_next = in_tile || (LA >= 1 && i + 1 < tb);
-            if (have_next) scores(nxt, ka);
-            float psum = 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                float pv = fast_exp2(__builtin_fmaf(cur[r], scale, -m_use));
-                cur[r] = pv;
-                psum += pv;
-            }
-            l_run += psum;
-            __builtin_amdgcn_sched_barrier(0);
-            // K operands of the step after next, behind the score MFMAs that read the old ones
-            if (kb + 2 < KB) {
-                load_k_operands(ka, stage, kb + 2);
-            } else if (KB > 1 && LA >= 1 && i + 1 < tb) {
-                load_k_operands(ka, stage_next, kb + 2 - KB);
-            }
-            accumulate(cur, vo, stage, kb);
-            if (have_next) mx_cur = in_tile ? prepare(nxt, full, k0 + 32 * (kb + 1)) : prepare(nxt, full_next, k0 + TK);
-        }
+        for (int kb = 0; kb < KB; kb++) step(stage, stage_next, kb, full, full_next, k0);
         if (KB & 1) s[0] = s[1];  // odd step count: the prefetched scores sit in the other buffer
     }
 
