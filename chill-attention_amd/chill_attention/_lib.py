@@ -11,7 +11,8 @@ import os
 from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_uint8, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libchill_attention_hip.so")
+# CHILL_ATTENTION_LIB names another build of the same library (for A/B measurements)
+LIB_PATH = os.environ.get("CHILL_ATTENTION_LIB") or os.path.join(os.path.dirname(_PKG_DIR), "lib", "libchill_attention_hip.so")
 
 ABI_VERSION = 1
 

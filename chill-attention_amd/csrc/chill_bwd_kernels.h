@@ -16,9 +16,15 @@
 //        dV^T += dO^T P, dK^T += Q^T dS, finally dK *= sm_scale        (chill_bwd_dkdv.py:362-403, 230)
 #pragma once
 
+#include <type_traits>
+
 #include "chill_device.h"
 #include "chill_params.h"
 #include "chill_tiles.h"
+
+#ifndef CHILL_SCHED_GROUPS
+#define CHILL_SCHED_GROUPS 0
+#endif
 
 namespace chill {
 
@@ -342,31 +348,64 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
     AsyncSwizzledLoader<E, D, TQS, NT> load_q, load_do;
     load_q.init(p.sq.t, wave, lane);
     load_do.init(p.sdo.t, wave, lane);
-    // iteration it = (group head g, q-tile)
-    auto issue_iter = [&](int it, int st_index) {
-        const int g = it / n_tiles;
-        const int q0 = (wg.start + it % n_tiles) * TQS;
+    // Iterations run over (group head g, q-tile).  The tile to issue next is tracked incrementally —
+    // pointers advance by one tile, and are rebuilt only when the next query head starts — so that
+    // issuing costs a handful of scalar instructions per iteration.
+    struct {
+        const ET* q;
+        const ET* d_o;
+        const float* lse;
+        const float* del;
+        int rows_left;  // rows from the tile's first row to the end of the tensor
+        int tile;       // index inside [0, n_tiles)
+        int g;
+    } nxt;
+    auto start_head = [&](int g) {
         const int hq = hkv * p.group + g;
+        const int q0 = wg.start * TQS;
+        nxt.q = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h + (int64_t)q0 * p.sq.t;
+        nxt.d_o = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h + (int64_t)q0 * p.sdo.t;
+        nxt.lse = p.lse + b * p.lse_b + hq * p.lse_h + q0;
+        nxt.del = p.delta + b * p.delta_b + hq * p.delta_h + q0;
+        nxt.rows_left = p.T - q0;
+        nxt.tile = 0;
+        nxt.g = g;
+    };
+    int n_issued = 0;
+    // move to the tile after the one just issued; past the end the last tile stays selected
+    auto advance = [&]() {
+        n_issued++;
+        if (n_issued >= n_iters) return;
+        if (nxt.tile + 1 == n_tiles) {
+            start_head(nxt.g + 1);
+        } else {
+            nxt.q += TQS * p.sq.t;
+            nxt.d_o += TQS * p.sdo.t;
+            nxt.lse += TQS;
+            nxt.del += TQS;
+            nxt.rows_left -= TQS;
+            nxt.tile++;
+        }
+    };
+    auto issue_next = [&](int st_index) {
         char* st = smem + RING_OFF + st_index * STAGE_BYTES;
-        const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
-        const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
-        load_q.issue(qptr + (int64_t)q0 * p.sq.t, p.T - q0, st, wave, lane);
-        load_do.issue(doptr + (int64_t)q0 * p.sdo.t, p.T - q0, st + TILE_BYTES, wave, lane);
+        load_q.issue(nxt.q, nxt.rows_left, st, wave, lane);
+        load_do.issue(nxt.d_o, nxt.rows_left, st + TILE_BYTES, wave, lane);
         if (wave == NW - 1) {
             // LSE2 and delta of the tile's rows; rows past the end of the tensor read as zero
-            const float* lse = p.lse + b * p.lse_b + hq * p.lse_h + q0;
-            const float* del = p.delta + b * p.delta_b + hq * p.delta_h + q0;
             char* vec = st + 2 * TILE_BYTES;
-            if (q0 + lane < p.T) {
-                async_load4(lse, lane * 4, lds_address(vec));
-                async_load4(del, lane * 4, lds_address(vec + VEC_BYTES));
+            if (lane < nxt.rows_left) {
+                async_load4(nxt.lse, lane * 4, lds_address(vec));
+                async_load4(nxt.del, lane * 4, lds_address(vec + VEC_BYTES));
             } else {
                 reinterpret_cast<float*>(vec)[lane] = 0.f;
                 reinterpret_cast<float*>(vec + VEC_BYTES)[lane] = 0.f;
             }
         }
+        advance();
     };
-    if (n_iters > 0) issue_iter(0, 0);
+    start_head(0);
+    if (n_iters > 0) issue_next(0);
 
     const int kw = kb0 + 32 * kblk;
     const int k_pos = kw + n;
@@ -387,6 +426,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
             dv[i][r] = 0.f;
         }
     const float scale = p.scale_log2;
+    const float masked_score = scale < 0.f ? INFINITY : -INFINITY;  // times the scale: -inf
     const lds_char* lds0 = (const lds_char*)smem;
     const lds_char* k_tile = lds0;
     const lds_char* v_tile = lds0 + KV_BYTES;
@@ -398,7 +438,14 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         __syncthreads();
         st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
         tile = tile + 1 == n_tiles ? 0 : tile + 1;
-        if (it + 1 < n_iters) issue_iter(it + 1, st_cur + 1 == NS ? 0 : st_cur + 1);
+        const int st_next = st_cur + 1 == NS ? 0 : st_cur + 1;
+        const bool in_block = !(tile < ta || tile >= tb);
+        // the two waves that share a SIMD issue their loads at different points of the iteration, so
+        // that one of them keeps the matrix pipe busy while the other sits in the memory pipeline
+        const bool issue_late = in_block && half == 1;
+        if (!issue_late) {
+            if (it + 1 < n_iters) issue_next(st_next);
+        }
         if (tile < ta || tile >= tb) continue;
         const lds_char* q_tile = lds0 + RING_OFF + st_cur * STAGE_BYTES;
         const lds_char* do_tile = q_tile + TILE_BYTES;
@@ -406,7 +453,17 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         const bool full = (tile >= fa) && (tile < fb);
         const int q0 = (wg.start + tile) * TQS + 32 * half;
 
-        // S = Q K^T, dP = dO V^T: both operands from LDS
+        // One 32 x 32 block.  The vector work is split in two parts, each placed among the MFMAs of a
+        // GEMM that does not depend on it: P = exp2(S * scale - LSE2) among the MFMAs of dP = dO V^T,
+        // dS = P (dP - delta) among those of dV^T += dO^T P.  All MFMA operands come from LDS.
+        // Masked entries get a score of -inf (times the sign of the scale) in a branch of their own, so
+        // that the rest of the block is the same straight-line code for full and partial tiles.
+        f32x4 lse4[4], del4[4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+            lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
+            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
+        }
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -416,29 +473,57 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
             s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
-            dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
         }
-        f32x4 lse4[4], del4[4];
+        if (!full) {
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-            lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
-            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
+            for (int r = 0; r < 16; r++) {
+                const int q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
+                const bool ok = (q < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(q, k_pos, seq_len, p.margs);
+                s[r] = ok ? s[r] : masked_score;
+                // a row that attends to nothing has LSE2 = -inf and only masked entries
+                const float l = lse4[r / 4][r % 4];
+                lse4[r / 4][r % 4] = (l == -INFINITY) ? 0.f : l;
+            }
         }
-        auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
-            q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
-            k = k_pos;
-            lse = lse4[r / 4][r % 4];
-            delta = del4[r / 4][r % 4];
-        };
-        if (full)
-            softmax_grad_block<MASK, false>(s, dp, scale, seq_len, p.margs, pos);
-        else
-            softmax_grad_block<MASK, true>(s, dp, scale, seq_len, p.margs, pos);
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+            dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
         mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);  // dV^T += dO^T P
+        if (issue_late) {
+            if (it + 1 < n_iters) issue_next(st_next);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) dp[r] = s[r] * (dp[r] - del4[r / 4][r % 4]);
         mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);  // dK^T += Q^T dS
+        if constexpr (Elem<E>::k16 && CHILL_SCHED_GROUPS) {
+            // one slot per MFMA: the MFMA, the two LDS reads of the NEXT MFMA's operands, a share of
+            // the vector work
+            constexpr int kValu = 0x402;  // vector ALU including transcendentals
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(kValu, (40 + NJ - 1) / NJ, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 2 * DB; j++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(kValu, (40 + 2 * DB - 1) / (2 * DB), 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 2 * DB; j++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (j + 1 < 2 * DB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            }
+        }
     }
 
     // sum the two waves of a pair through LDS (one accumulator at a time), then store
+    wait_async_tiles();
     float* red = reinterpret_cast<float*>(smem) + kblk * (DB * 16 * 64) + lane;
     auto reduce_and_store = [&](f32x16 (&acc)[DB], ET* base, int64_t row_stride, float mult) {
         __syncthreads();  // everyone is done with the tiles (or with the previous round)
