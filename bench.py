@@ -121,9 +121,10 @@ class Runner:
         return ks
 
 
-def cpu_baseline(torch, mask_name, margs, dtype_name, T, D, mode, seed, sigma, budget_s=20.0):
+def cpu_baseline(torch, mask_name, margs, dtype_name, T, D, mode, seed, sigma, budget_s=15.0):
     """Reference CPU path on a bounded sample: dense mask -> torch SDPA (fp32 on upcast inputs, as
-    the reference's tests run it), one (batch, head) slice of the workload at full T per call."""
+    the reference's tests run it), one (batch, head) slice of the workload at full T per call,
+    repeated for about budget_s seconds (at least 3 calls, at most 64)."""
     sys.path.insert(0, ROOT)
     from oracle import chill_oracle as orc
 
@@ -144,7 +145,8 @@ def cpu_baseline(torch, mask_name, margs, dtype_name, T, D, mode, seed, sigma, b
         if mode == "fwd+bwd":
             out.backward(do)
         times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_begin > budget_s or len(times) >= 4:
+        elapsed = time.perf_counter() - t_begin
+        if (elapsed > budget_s and len(times) >= 3) or len(times) >= 64 or elapsed > 4 * budget_s:
             break
     used = times[1:] if len(times) > 1 else times  # the first run warms the allocator up
     timed = len(used)
