@@ -460,10 +460,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         // that the rest of the block is the same straight-line code for full and partial tiles.
         f32x4 lse4[4], del4[4];
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
+        for (int g4 = 0; g4 < 4; g4++)
             lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
-            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
-        }
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -490,6 +488,9 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
             dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++)
+            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
         mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);  // dV^T += dO^T P
         if (issue_late) {
             if (it + 1 < n_iters) issue_next(st_next);
