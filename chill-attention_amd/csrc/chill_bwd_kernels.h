@@ -22,10 +22,6 @@
 #include "chill_params.h"
 #include "chill_tiles.h"
 
-#ifndef CHILL_SCHED_GROUPS
-#define CHILL_SCHED_GROUPS 0
-#endif
-
 namespace chill {
 
 // ------------------------------------------------------------------------------------------ delta
@@ -453,9 +449,9 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         const bool full = (tile >= fa) && (tile < fb);
         const int q0 = (wg.start + tile) * TQS + 32 * half;
 
-        // One 32 x 32 block.  The vector work is split in two parts, each placed among the MFMAs of a
-        // GEMM that does not depend on it: P = exp2(S * scale - LSE2) among the MFMAs of dP = dO V^T,
-        // dS = P (dP - delta) among those of dV^T += dO^T P.  All MFMA operands come from LDS.
+        // One 32 x 32 block.  The vector work is split in two parts, each written next to a GEMM that
+        // does not depend on it: P = exp2(S * scale - LSE2) after dP = dO V^T has been issued,
+        // dS = P (dP - delta) after dV^T += dO^T P.  All MFMA operands come from LDS.
         // Masked entries get a score of -inf (times the sign of the scale) in a branch of their own, so
         // that the rest of the block is the same straight-line code for full and partial tiles.
         f32x4 lse4[4], del4[4];
@@ -498,29 +494,6 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
 #pragma unroll
         for (int r = 0; r < 16; r++) dp[r] = s[r] * (dp[r] - del4[r / 4][r % 4]);
         mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);  // dK^T += Q^T dS
-        if constexpr (Elem<E>::k16 && CHILL_SCHED_GROUPS) {
-            // one slot per MFMA: the MFMA, the two LDS reads of the NEXT MFMA's operands, a share of
-            // the vector work
-            constexpr int kValu = 0x402;  // vector ALU including transcendentals
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-#pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(kValu, (40 + NJ - 1) / NJ, 0);
-            }
-#pragma unroll
-            for (int j = 0; j < 2 * DB; j++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                __builtin_amdgcn_sched_group_barrier(kValu, (40 + 2 * DB - 1) / (2 * DB), 0);
-            }
-#pragma unroll
-            for (int j = 0; j < 2 * DB; j++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (j + 1 < 2 * DB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-            }
-        }
     }
 
     // sum the two waves of a pair through LDS (one accumulator at a time), then store

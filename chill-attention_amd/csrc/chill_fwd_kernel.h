@@ -32,9 +32,6 @@ namespace chill {
 
 // Lazy-rescale threshold of the online softmax, in log2 units: P stays below 2^kRescaleTau.
 constexpr float kRescaleTau = 8.0f;
-#ifndef CHILL_SCHED_GROUPS
-#define CHILL_SCHED_GROUPS 1
-#endif
 
 template <typename E, int D, int TK>
 struct FwdLds {
@@ -237,8 +234,8 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
     // One step: softmax of the current 32-key block and its share of O, with the scores of the next
     // block issued first.  With a tile resident ahead (LA >= 1) the step reads the next block
     // unconditionally — a wave's last step reads a stage whose contents it never uses — so that
-    // between the rare rescale branch and the mask branch the step is one basic block in which
-    // the instruction groups below interleave matrix and vector work.
+    // between the rare rescale branch and the mask branch the step is one basic block, in which the
+    // compiler places the softmax of this step among the score MFMAs of the next.
     auto step = [&](const lds_char* stage, const lds_char* stage_next, int kb, bool full, bool full_next, int k0) {
         f32x16& cur = s[kb & 1];
         f32x16& nxt = s[(kb + 1) & 1];
@@ -273,16 +270,6 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
             psum += pv;
         }
         l_run += psum;
-        if constexpr (Elem<E>::k16 && CHILL_SCHED_GROUPS) {
-            // every score MFMA is followed by its share of the softmax
-            if (have_next) {
-#pragma unroll
-                for (int j = 0; j < NJ; j++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x402, (48 + NJ - 1) / NJ, 0);
-                }
-            }
-        }
         __builtin_amdgcn_sched_barrier(0);
         // K operands of the step after next, behind the score MFMAs that read the old ones
         if (kb + 2 < KB) {

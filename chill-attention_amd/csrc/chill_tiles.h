@@ -10,13 +10,6 @@
 
 #include "chill_params.h"
 
-#ifndef CHILL_FWD_TK
-#define CHILL_FWD_TK 64
-#endif
-#ifndef CHILL_DQ_TK
-#define CHILL_DQ_TK 64
-#endif
-
 namespace chill {
 
 constexpr int elem_bytes(int dtype) { return dtype == CHILL_F32 ? 4 : 2; }
@@ -39,7 +32,7 @@ constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
     const int waves = fast16 ? 8 : 4;
-    const int streamed = fast16 ? CHILL_FWD_TK : 32;
+    const int streamed = fast16 ? 64 : 32;
     return TileConfig{waves * 32, streamed, waves,
                       fwd_stages_for(streamed, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
 }
@@ -53,7 +46,7 @@ constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
     const int waves = fast16 ? 8 : 4;
-    const int streamed = fast16 ? CHILL_DQ_TK : 32;
+    const int streamed = fast16 ? 64 : 32;
     return TileConfig{waves * 32, streamed, waves,
                       dq_stages_for(streamed, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
 }
