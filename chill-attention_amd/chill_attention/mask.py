@@ -250,6 +250,105 @@ class ChillMask(ABC):
         """FlexAttention ``BlockMask`` of the same pattern, or None (reference mask.py:473-483)."""
         return None
 
+    def _calc_full_ranges(self, max_pos: int, TILE_Q: int) -> torch.Tensor:
+        """``[n_tiles, 2]`` int32: the half-open predicate-free key range of every query tile
+        (reference mask.py:507-534)."""
+        n_tiles = -(-max_pos // TILE_Q)
+        out = np.zeros((n_tiles, 2), dtype=np.int32)
+        for i in range(n_tiles):
+            lo, hi = self.k_full_range_for_q(i * TILE_Q, TILE_Q, max_pos, self.constargs)
+            out[i] = (int(lo), int(hi))
+        return torch.from_numpy(out)
+
+    def plot(
+        self,
+        max_pos,
+        draw_full_blocks: typing.Union[bool, int, typing.Tuple[int, int]] = False,
+        plot_block_types: bool = False,
+        TILE_Q: int = 32,
+        TILE_K: int = 32,
+    ):
+        """Draw the mask (reference mask.py:536-698): left panel rows = queries, right panel its
+        transpose, each with the analytical limits of the streamed axis drawn over it.
+
+        Args:
+            max_pos: number of positions to draw.
+            draw_full_blocks: outline the blocks ``is_full_block`` reports — ``True`` for tile sizes
+                16..256, an int for one square tile size, a pair for one ``(q, k)`` tile size.
+            plot_block_types: shade, per query tile of ``TILE_Q`` rows, the key range that the
+                kernels run without predicate (``k_full_range_for_q``).
+            TILE_Q, TILE_K: tile sizes for ``plot_block_types``.
+
+        Returns:
+            matplotlib.figure.Figure
+        """
+        import itertools
+
+        import matplotlib
+
+        if not matplotlib.get_backend():
+            matplotlib.use("Agg")
+        import matplotlib.patches as patches
+        import matplotlib.pyplot as plt
+
+        dense = self.make_mask(max_pos).cpu().numpy()
+        k_lims = self._calc_limits(max_pos, 0).numpy()  # per query: [lo, hi] over keys
+        q_lims = self._calc_limits(max_pos, 1).numpy()  # per key: [lo, hi] over queries
+        pos = np.arange(max_pos)
+
+        fig, axes = plt.subplots(1, 2, figsize=(10, 5))
+        panels = (
+            (axes[0], dense, q_lims, "k index", "q index", "q_lims_for_k"),
+            (axes[1], dense.T, k_lims, "q index", "k index", "k_lims_for_q"),
+        )
+        for ax, image, lims, xlabel, ylabel, what in panels:
+            ax.imshow(image, origin="lower", vmin=0, vmax=1)
+            ax.plot(pos, np.clip(lims[:, 0] - 0.5, -0.5, max_pos - 1), color="red", label=f"min {what}")
+            ax.plot(pos, np.clip(lims[:, 1] + 0.5, -0.5, max_pos - 1), color="blue", label=f"max {what}")
+            ax.set_xlabel(xlabel)
+            ax.set_ylabel(ylabel)
+
+        if draw_full_blocks:
+            if isinstance(draw_full_blocks, bool):
+                sizes_q = sizes_k = [16, 32, 64, 128, 256]
+            elif isinstance(draw_full_blocks, int):
+                sizes_q = sizes_k = [draw_full_blocks]
+            else:
+                sizes_q, sizes_k = [draw_full_blocks[0]], [draw_full_blocks[1]]
+            styles = itertools.cycle(
+                itertools.product(["black", "green", "violet", "purple", "darkorange", "white", "lightblue"], ["-", "--", ":"])
+            )
+            for tq in sizes_q:
+                for tk in sizes_k:
+                    if not self.has_full_blocks(tq, tk, seq_len=max_pos, args=self.constargs):
+                        continue
+                    color, style = next(styles)
+                    for q, k in self._calc_full_block_indices(max_pos, tq, tk):
+                        if q + tq > max_pos or k + tk > max_pos or not dense[q : q + tq, k : k + tk].any():
+                            continue
+                        for ax, (x, y, w, h) in zip(axes, ((k, q, tk, tq), (q, k, tq, tk))):
+                            ax.add_patch(
+                                patches.Rectangle((x - 0.5, y - 0.5), w, h, ls=style, ec=color, zorder=2, alpha=0.3, fill=False)
+                            )
+
+        if plot_block_types and self.has_k_full_range():
+            full_ranges = self._calc_full_ranges(max_pos, TILE_Q).numpy()
+            first = True
+            for i, (ks, ke) in enumerate(full_ranges):
+                if ke <= ks:
+                    continue
+                qb = i * TILE_Q
+                style = dict(color="yellow", alpha=0.6, zorder=4, ec="red", ls="-", lw=1.5)
+                axes[0].add_patch(
+                    patches.Rectangle((ks - 0.5, qb - 0.5), ke - ks, TILE_Q, label="predicate-free range" if first else None, **style)
+                )
+                axes[1].add_patch(patches.Rectangle((qb - 0.5, ks - 0.5), TILE_Q, ke - ks, **style))
+                first = False
+
+        axes[0].legend()
+        axes[1].legend()
+        return fig
+
 
 _DESC_IDS: dict = {}
 
@@ -618,3 +717,14 @@ class PrefixLMChillMask(ChillMask):
     def make_flex_mask(self, max_pos):
         prefix = self.constargs[0]
         return _flex(lambda b, h, q, k: (k < prefix) | (q >= k), max_pos)
+
+
+if __name__ == "__main__":
+    # python -m chill_attention.mask: draw a mask and check its rules (reference mask.py:1397-1407)
+    import matplotlib
+
+    matplotlib.use("Agg")
+    demo = SlidingWindowChillMask(10, 4)
+    demo.plot(200, True).savefig("mask.png")
+    demo.verify(1024)
+    print(f"{demo}: rules verified up to 1024 positions, drawing in mask.png")

@@ -172,3 +172,23 @@ def test_flex_mask_consistent(m):
     assert flex is not None
     dense = create_mask(flex.mask_mod, None, None, n, n, device=mask.make_mask(1).device)[0, 0]
     assert (dense.cpu() == mask.make_mask(n).cpu()).all()
+
+
+def test_plot_draws_both_panels(tmp_path):
+    """plot() (reference mask.py:536-698) returns a two-panel figure; full blocks and predicate-free
+    ranges are drawn as patches."""
+    import matplotlib
+
+    matplotlib.use("Agg")
+    m = ca.SlidingWindowChillMask(40, 8)
+    fig = m.plot(96, draw_full_blocks=16, plot_block_types=True, TILE_Q=16, TILE_K=16)
+    assert len(fig.axes) == 2
+    assert all(len(ax.lines) == 2 for ax in fig.axes)
+    assert len(fig.axes[0].patches) > 0 and len(fig.axes[0].patches) == len(fig.axes[1].patches)
+    fig.savefig(tmp_path / "mask.png")
+    assert (tmp_path / "mask.png").stat().st_size > 0
+    full = m._calc_full_ranges(96, 16).numpy()
+    dense = m.make_mask(96).cpu().numpy()
+    for i, (lo, hi) in enumerate(full):
+        if hi > lo:
+            assert dense[16 * i : 16 * i + 16, lo:hi].all()
