@@ -19,6 +19,7 @@ ABI_VERSION = 1
 # ChillDType / ChillMaskId / ChillPass of the header
 F32, F16, BF16 = 0, 1, 2
 MASK_FULL, MASK_CAUSAL, MASK_SLIDING_WINDOW, MASK_CHUNKWISE, MASK_PREFIX_LM = range(5)
+MASK_USER = 5  # the one mask of a library built around a user-written functor
 PASS_FWD, PASS_DQ, PASS_DKDV = 0, 1, 2
 
 
@@ -38,14 +39,16 @@ class ChillLibraryError(RuntimeError):
         self.status = status
 
 
-def _load() -> ctypes.CDLL:
-    if not os.path.exists(LIB_PATH):
+def load_library(path: str) -> ctypes.CDLL:
+    """Load one build of the library (the stock one, or one built around a user mask) and declare
+    the C ABI on it."""
+    if not os.path.exists(path):
         raise ImportError(
-            f"chill_attention: the HIP library {LIB_PATH} has not been built "
+            f"chill_attention: the HIP library {path} has not been built "
             "(run `make -C chill-attention_amd/csrc -j8` or `python -c 'import __graft_entry__ as g; g.build()'`). "
             "There is no fallback implementation."
         )
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     P = POINTER
     T4 = P(ChillTensor4)
     MD = P(ChillMaskDesc)
@@ -69,6 +72,7 @@ def _load() -> ctypes.CDLL:
         "chill_mask_nnz": (c_int64, [MD, c_int32]),
         "chill_status_string": (c_char_p, [c_int32]),
         "chill_abi_version": (c_int32, []),
+        "chill_has_user_mask": (c_int32, []),
     }
     for name, (restype, argtypes) in sig.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
@@ -80,12 +84,12 @@ def _load() -> ctypes.CDLL:
     return lib
 
 
-lib = _load()
+lib = load_library(LIB_PATH)
 EXPORTED_SYMBOLS = (
     "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dkdv", "chill_mask_eval_device",
     "chill_tile_ranges_device", "chill_mask_eval", "chill_mask_limits", "chill_tile_ranges",
     "chill_mask_is_full_block", "chill_mask_has_full_blocks", "chill_tile_config", "chill_mask_nnz",
-    "chill_status_string", "chill_abi_version",
+    "chill_status_string", "chill_abi_version", "chill_has_user_mask",
 )
 
 

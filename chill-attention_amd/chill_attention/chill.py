@@ -74,6 +74,10 @@ def register_chill_mask(mask: ChillMask):
         return
     mask_cls = type(mask)
 
+    # the library that holds this class's functor (a user-written mask has one of its own, built
+    # here on first registration)
+    mask_lib = mask_cls._library()
+
     def mask_cls_descriptor(mask_args):
         return _descriptor(mask_cls, tuple(mask_args))
 
@@ -104,7 +108,7 @@ def register_chill_mask(mask: ChillMask):
         lens_ptr, lens_stride = _lens_args(lens)
         tq, tk, tv, to = _lib.tensor4(qv), _lib.tensor4(kv), _lib.tensor4(vv), _lib.tensor4(O)
         with torch.cuda.device(q.device):
-            status = _lib.lib.chill_fwd(
+            status = mask_lib.chill_fwd(
                 ctypes.byref(tq), ctypes.byref(tk), ctypes.byref(tv), ctypes.byref(to),
                 ctypes.c_void_p(LSE.data_ptr()) if LSE is not None else None,
                 _lib.strides3(LSE) if LSE is not None else None,
@@ -165,14 +169,14 @@ def register_chill_mask(mask: ChillMask):
         with torch.cuda.device(q.device):
             _lib.check(
                 "chill_bwd_delta",
-                _lib.lib.chill_bwd_delta(
+                mask_lib.chill_bwd_delta(
                     ctypes.byref(to), ctypes.byref(tdo), delta_p, _lib.strides3(delta),
                     batch, heads, T, head_dim, dtype, stream,
                 ),
             )
             _lib.check(
                 "chill_bwd_dkdv",
-                _lib.lib.chill_bwd_dkdv(
+                mask_lib.chill_bwd_dkdv(
                     ctypes.byref(tq), ctypes.byref(tk), ctypes.byref(tv), ctypes.byref(tdo),
                     ctypes.byref(tdk), ctypes.byref(tdv),
                     lse_p, _lib.strides3(lse), delta_p, _lib.strides3(delta), lens_ptr, lens_stride,
@@ -182,7 +186,7 @@ def register_chill_mask(mask: ChillMask):
             )
             _lib.check(
                 "chill_bwd_dq",
-                _lib.lib.chill_bwd_dq(
+                mask_lib.chill_bwd_dq(
                     ctypes.byref(tq), ctypes.byref(tk), ctypes.byref(tv), ctypes.byref(tdo), ctypes.byref(tdq),
                     lse_p, _lib.strides3(lse), delta_p, _lib.strides3(delta), lens_ptr, lens_stride,
                     batch, heads, num_kv_heads, T, head_dim, dtype, float(sm_scale),

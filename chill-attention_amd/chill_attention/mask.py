@@ -118,6 +118,14 @@ class ChillMask(ABC):
         """The mask-id + args descriptor handed to the C ABI."""
         return _descriptor(type(self), self.constargs)
 
+    @classmethod
+    def _library(cls):
+        """The loaded library that holds this class's functor: the stock one for the built-in masks,
+        a library of its own (built on first use, see ``user_mask``) for a user-written mask."""
+        from . import user_mask
+
+        return user_mask.library_for(cls) if user_mask.is_user_mask(cls) else _lib.lib
+
     # ------------------------------------------------------------------ enumeration
     def make_mask(self, max_pos: int) -> torch.Tensor:
         """Dense boolean mask ``[max_pos, max_pos]`` (rows = queries), reference mask.py:379-412.
@@ -127,7 +135,7 @@ class ChillMask(ABC):
         desc = self.descriptor()
         _lib.check(
             "chill_mask_eval",
-            _lib.lib.chill_mask_eval(ctypes.byref(desc), max_pos, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))),
+            self._library().chill_mask_eval(ctypes.byref(desc), max_pos, out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))),
         )
         return torch.from_numpy(out).to(torch.bool).to(_best_device())
 
@@ -140,7 +148,7 @@ class ChillMask(ABC):
         desc = self.descriptor()
         _lib.check(
             "chill_mask_limits",
-            _lib.lib.chill_mask_limits(
+            self._library().chill_mask_limits(
                 ctypes.byref(desc), which, max_pos, total_pos, out.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
             ),
         )
@@ -157,7 +165,7 @@ class ChillMask(ABC):
         desc = self.descriptor()
         _lib.check(
             "chill_tile_ranges",
-            _lib.lib.chill_tile_ranges(
+            self._library().chill_tile_ranges(
                 ctypes.byref(desc), pass_id, max_pos, seq_len, tile_in, tile_out,
                 out.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)),
             ),
@@ -175,7 +183,7 @@ class ChillMask(ABC):
     def nnz(self, max_pos: int) -> int:
         """Number of unmasked (q, k) pairs below ``max_pos`` (effective-FLOP numerator)."""
         desc = self.descriptor()
-        return int(_lib.check("chill_mask_nnz", _lib.lib.chill_mask_nnz(ctypes.byref(desc), max_pos)))
+        return int(_lib.check("chill_mask_nnz", self._library().chill_mask_nnz(ctypes.byref(desc), max_pos)))
 
     def verify(self, max_pos: int):
         """Check every rule of the mask against brute-force enumeration of the dense mask.
@@ -354,15 +362,21 @@ _DESC_IDS: dict = {}
 
 
 def _descriptor(cls, constargs) -> "_lib.ChillMaskDesc":
-    if cls.mask_id is None:
-        raise NotImplementedError(
-            f"{cls.__name__} has no compiled functor in the HIP library; only the built-in masks "
-            "(Full, Causal, SlidingWindow, Chunkwise, PrefixLM) lower to a mask id"
-        )
+    from . import user_mask
+
+    mask_id = cls.mask_id
+    if mask_id is None:
+        if not user_mask.is_user_mask(cls):
+            raise NotImplementedError(
+                f"{cls.__name__} has no compiled functor: the built-in masks (Full, Causal, SlidingWindow, "
+                "Chunkwise, PrefixLM) lower to a mask id, a mask of your own needs a `hip_functor` "
+                "(see chill_attention.user_mask)"
+            )
+        mask_id = _lib.MASK_USER
     for a in constargs:
         if isinstance(a, float) and not float(a).is_integer():
             raise ValueError(f"{cls.__name__}: mask arguments must be integers, got {a!r}")
-    return _lib.mask_desc(cls.mask_id, [int(a) for a in constargs])
+    return _lib.mask_desc(mask_id, [int(a) for a in constargs])
 
 
 def _flex(mask_mod, max_pos):

@@ -23,9 +23,10 @@ def tile_config(mask, head_dim: int, dtype: torch.dtype, pass_id: int) -> dict:
     workgroup and LDS bytes per workgroup.
     """
     out = (ctypes.c_int32 * 4)()
+    mask_id = mask.mask_id if mask.mask_id is not None else _lib.MASK_USER
     _lib.check(
         "chill_tile_config",
-        _lib.lib.chill_tile_config(mask.mask_id, head_dim, _DTYPES[dtype], pass_id, out),
+        mask._library().chill_tile_config(mask_id, head_dim, _DTYPES[dtype], pass_id, out),
     )
     return {"rows": out[0], "streamed": out[1], "waves": out[2], "lds_bytes": out[3]}
 

@@ -100,12 +100,18 @@ int64_t chill_mask_nnz(const ChillMaskDesc* mask, int32_t T) {
     int st = lower_mask(mask, &a);
     if (st != CHILL_OK) return st;
     if (T < 0) return CHILL_ERR_BAD_SHAPE;
-    // every built-in mask row is one interval [lo, hi] of keys, so the count is a sum of lengths
+    // every built-in mask row is one interval [lo, hi] of keys, so the count is a sum of lengths;
+    // a user mask may have holes inside its limits and is counted position by position
     int64_t total = 0;
     CHILL_DISPATCH_MASK(mask->id, {
         for (int q = 0; q < T; q++) {
             Range r = Mask<MASK_ID>::k_range_for_q(q, T, a);
-            if (r.hi >= r.lo) total += (int64_t)(r.hi - r.lo + 1);
+            if (r.hi < r.lo) continue;
+            if (MASK_ID == CHILL_MASK_USER) {
+                for (int k = r.lo; k <= r.hi; k++) total += Mask<MASK_ID>::pred(q, k, T, a) ? 1 : 0;
+            } else {
+                total += (int64_t)(r.hi - r.lo + 1);
+            }
         }
     });
     return total;
@@ -113,7 +119,7 @@ int64_t chill_mask_nnz(const ChillMaskDesc* mask, int32_t T) {
 
 int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int32_t out[4]) {
     if (out == nullptr) return CHILL_ERR_NULL_POINTER;
-    if (mask_id < 0 || mask_id >= CHILL_MASK_COUNT) return CHILL_ERR_BAD_MASK;
+    if (!mask_id_served(mask_id)) return CHILL_ERR_BAD_MASK;
     TileConfig c;
     int st = tile_config(mask_id, D, dtype, pass, &c);
     if (st != CHILL_OK) return st;
@@ -141,5 +147,13 @@ const char* chill_status_string(int32_t status) {
 }
 
 int32_t chill_abi_version(void) { return CHILL_ABI_VERSION; }
+
+int32_t chill_has_user_mask(void) {
+#ifdef CHILL_USER_MASK_HEADER
+    return 1;
+#else
+    return 0;
+#endif
+}
 
 }  // extern "C"

@@ -25,6 +25,8 @@ namespace chill {
 struct MaskArgs {
     int a0;
     int a1;
+    int a2;
+    int a3;
 };
 
 struct Range {
@@ -44,9 +46,26 @@ CHILL_HD int floordiv(int a, int b) {
 template <int ID>
 struct Mask;
 
+// What a mask functor inherits unless it says otherwise — the defaults of the reference's ChillMask
+// base class (mask.py:110-250): no predicate-free ranges, no full blocks, rows may be empty, and
+// limits that never decrease from one row to the next (the reference's *_lims_continious = True).
+// A functor whose limits are NOT monotone sets kMonotoneLimits = false; tile ranges then come
+// from the minimum / maximum over the rows of a tile (utils.py:259-268).
+struct MaskDefaults {
+    static constexpr int kNumArgs = 0;
+    static constexpr bool kSafe = false;
+    static constexpr bool kHasKFullRange = false;
+    static constexpr bool kHasQFullRange = false;
+    static constexpr bool kMonotoneLimits = true;
+    CHILL_HD static Range k_full_range_for_q(int, int, int, MaskArgs) { return {0, 0}; }
+    CHILL_HD static Range q_full_range_for_k(int, int, int, MaskArgs) { return {0, 0}; }
+    CHILL_HD static bool has_full_blocks(int, int, int, MaskArgs) { return false; }
+    CHILL_HD static bool is_full_block(int, int, int, int, int, MaskArgs) { return false; }
+};
+
 // ---------------------------------------------------------------- Full (mask.py:806-889)
 template <>
-struct Mask<CHILL_MASK_FULL> {
+struct Mask<CHILL_MASK_FULL> : MaskDefaults {
     static constexpr int kNumArgs = 0;
     static constexpr bool kSafe = true;        // every row sees at least one key (mask.py:864)
     static constexpr bool kHasKFullRange = true;
@@ -62,7 +81,7 @@ struct Mask<CHILL_MASK_FULL> {
 
 // ---------------------------------------------------------------- Causal (mask.py:892-976)
 template <>
-struct Mask<CHILL_MASK_CAUSAL> {
+struct Mask<CHILL_MASK_CAUSAL> : MaskDefaults {
     static constexpr int kNumArgs = 0;
     static constexpr bool kSafe = true;
     static constexpr bool kHasKFullRange = true;
@@ -85,7 +104,7 @@ struct Mask<CHILL_MASK_CAUSAL> {
 // ---------------------------------------------------------------- SlidingWindow (mask.py:979-1108)
 // args: a0 = left_context, a1 = right_context
 template <>
-struct Mask<CHILL_MASK_SLIDING_WINDOW> {
+struct Mask<CHILL_MASK_SLIDING_WINDOW> : MaskDefaults {
     static constexpr int kNumArgs = 2;
     static constexpr bool kSafe = false;
     static constexpr bool kHasKFullRange = true;
@@ -128,7 +147,7 @@ struct Mask<CHILL_MASK_SLIDING_WINDOW> {
 // ---------------------------------------------------------------- Chunkwise (mask.py:1111-1266)
 // args: a0 = context_size (> 0), a1 = back_contexts (>= 0)
 template <>
-struct Mask<CHILL_MASK_CHUNKWISE> {
+struct Mask<CHILL_MASK_CHUNKWISE> : MaskDefaults {
     static constexpr int kNumArgs = 2;
     static constexpr bool kSafe = false;
     static constexpr bool kHasKFullRange = true;
@@ -175,7 +194,7 @@ struct Mask<CHILL_MASK_CHUNKWISE> {
 // ---------------------------------------------------------------- PrefixLM (mask.py:1269-1394)
 // args: a0 = prefix_size
 template <>
-struct Mask<CHILL_MASK_PREFIX_LM> {
+struct Mask<CHILL_MASK_PREFIX_LM> : MaskDefaults {
     static constexpr int kNumArgs = 1;
     static constexpr bool kSafe = true;
     static constexpr bool kHasKFullRange = true;
@@ -229,6 +248,20 @@ CHILL_HD TileRange tile_range(int i, int tile_in, int tile_out, int seq_len, boo
     int i_max = imin(i + tile_in, seq_len) - 1;
     Range first = QROWS ? M::k_range_for_q(i, seq_len, a) : M::q_range_for_k(i, seq_len, a);
     Range last = QROWS ? M::k_range_for_q(i_max, seq_len, a) : M::q_range_for_k(i_max, seq_len, a);
+    if (!M::kMonotoneLimits) {
+        // hull of the rows' ranges; rows without any visible position (hi < lo) do not count
+        int lo = 0x7fffffff, hi = -1;
+        for (int row = i; row <= i_max; row++) {
+            Range rr = QROWS ? M::k_range_for_q(row, seq_len, a) : M::q_range_for_k(row, seq_len, a);
+            if (rr.hi >= rr.lo) {
+                lo = imin(lo, rr.lo);
+                hi = imax(hi, rr.hi);
+            }
+        }
+        if (hi < 0) lo = 0;
+        first.lo = lo;
+        last.hi = hi;
+    }
     TileRange r;
     r.start = first.lo / tile_out;
     r.end = cdiv(last.hi + 1, tile_out);
@@ -259,7 +292,27 @@ CHILL_HD bool pass_has_full_blocks(bool qrows, int tile_in, int tile_out, int T,
                  : Mask<ID>::has_full_blocks(tile_out, tile_in, T, a);
 }
 
+}  // namespace chill
+
+// A library built with -DCHILL_USER_MASK_HEADER='"file"' compiles ONE extra functor, written by the
+// user, and serves only that one (so that the build stays a fifth of the stock one).  The file
+// specialises chill::Mask<CHILL_MASK_USER>; chill_user_mask.h documents what it must contain.
+#ifdef CHILL_USER_MASK_HEADER
+#include CHILL_USER_MASK_HEADER
+#endif
+
+namespace chill {
+
 // Runtime dispatch over the mask id for host-side entry points and launchers.
+#ifdef CHILL_USER_MASK_HEADER
+#define CHILL_DISPATCH_MASK(id, ...)                                                  \
+    switch (id) {                                                                     \
+        case CHILL_MASK_USER: { constexpr int MASK_ID = CHILL_MASK_USER; __VA_ARGS__; } break; \
+        default: break;                                                               \
+    }
+inline bool mask_id_served(int id) { return id == CHILL_MASK_USER; }
+inline int mask_num_args(int) { return Mask<CHILL_MASK_USER>::kNumArgs; }
+#else
 #define CHILL_DISPATCH_MASK(id, ...)                                                  \
     switch (id) {                                                                     \
         case CHILL_MASK_FULL: { constexpr int MASK_ID = CHILL_MASK_FULL; __VA_ARGS__; } break; \
@@ -269,13 +322,18 @@ CHILL_HD bool pass_has_full_blocks(bool qrows, int tile_in, int tile_out, int T,
         case CHILL_MASK_PREFIX_LM: { constexpr int MASK_ID = CHILL_MASK_PREFIX_LM; __VA_ARGS__; } break; \
         default: break;                                                               \
     }
+inline bool mask_id_served(int id) { return id >= 0 && id < CHILL_MASK_COUNT; }
+inline int mask_num_args(int id) {
+    static const int nargs[CHILL_MASK_COUNT] = {0, 0, 2, 2, 1};
+    return nargs[id];
+}
+#endif
 
 // Validates a descriptor and lowers it to kernel arguments.  Returns a ChillStatus.
 inline int lower_mask(const ChillMaskDesc* d, MaskArgs* out) {
     if (d == nullptr) return CHILL_ERR_NULL_POINTER;
-    if (d->id < 0 || d->id >= CHILL_MASK_COUNT) return CHILL_ERR_BAD_MASK;
-    static const int nargs[CHILL_MASK_COUNT] = {0, 0, 2, 2, 1};
-    if (d->nargs != nargs[d->id]) return CHILL_ERR_BAD_MASK;
+    if (!mask_id_served(d->id)) return CHILL_ERR_BAD_MASK;
+    if (d->nargs != mask_num_args(d->id) || d->nargs > 4) return CHILL_ERR_BAD_MASK;
     // arguments are position-like: keep sums with positions inside int32
     const int64_t kMaxArg = (int64_t)1 << 29;
     for (int i = 0; i < d->nargs; i++) {
@@ -283,6 +341,8 @@ inline int lower_mask(const ChillMaskDesc* d, MaskArgs* out) {
     }
     out->a0 = d->nargs > 0 ? (int)d->args[0] : 0;
     out->a1 = d->nargs > 1 ? (int)d->args[1] : 0;
+    out->a2 = d->nargs > 2 ? (int)d->args[2] : 0;
+    out->a3 = d->nargs > 3 ? (int)d->args[3] : 0;
     if (d->id == CHILL_MASK_CHUNKWISE) {
         if (out->a0 <= 0) return CHILL_ERR_BAD_MASK;
         // (chunk + back + 1) * context must stay inside int32 for T < 2^29

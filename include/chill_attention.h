@@ -49,14 +49,19 @@ typedef enum ChillDType {
     CHILL_BF16 = 2
 } ChillDType;
 
-/* Mask ids: one per ChillMask class of the reference (chill_attention/mask.py:806-1394). */
+/* Mask ids: one per ChillMask class of the reference (chill_attention/mask.py:806-1394), plus
+ * CHILL_MASK_USER for a library built around one user-written functor — the counterpart of the
+ * reference's "Creating Your Own Mask" (README.md:124-179; ChillMask contract mask.py:54-250).
+ * Such a library (make USER_MASK=functor.h, see csrc/chill_user_mask.h) serves ONLY
+ * CHILL_MASK_USER; the stock library serves only the five built-in ids. */
 typedef enum ChillMaskId {
     CHILL_MASK_FULL = 0,           /* FullChillMask            mask.py:806-889,   no args          */
     CHILL_MASK_CAUSAL = 1,         /* CausalChillMask          mask.py:892-976,   no args          */
     CHILL_MASK_SLIDING_WINDOW = 2, /* SlidingWindowChillMask   mask.py:979-1108,  (left, right)    */
     CHILL_MASK_CHUNKWISE = 3,      /* ChunkwiseChillMask       mask.py:1111-1266, (context, back)  */
     CHILL_MASK_PREFIX_LM = 4,      /* PrefixLMChillMask        mask.py:1269-1394, (prefix,)        */
-    CHILL_MASK_COUNT = 5
+    CHILL_MASK_COUNT = 5,          /* number of built-in masks */
+    CHILL_MASK_USER = 5            /* user-written functor, up to 4 integer args      */
 } ChillMaskId;
 
 /* The "mask-ID-plus-args" descriptor a ChillMask instance lowers to.  The reference bakes
@@ -182,6 +187,11 @@ int64_t chill_mask_nnz(const ChillMaskDesc* mask, int32_t T);
 
 const char* chill_status_string(int32_t status);
 int32_t chill_abi_version(void);
+
+/* 1 if this library was built around a user-written functor (it then serves CHILL_MASK_USER and
+ * nothing else), 0 for the stock library.  No counterpart in the reference, where a user mask is
+ * a Python class whose Triton methods are compiled on first use (chill.py:27-58). */
+int32_t chill_has_user_mask(void);
 
 #ifdef __cplusplus
 }

@@ -56,11 +56,14 @@ MASK_NAMES = (
 # --------------------------------------------------------------------------------------------
 # mask predicate — two independent statements
 # --------------------------------------------------------------------------------------------
-def mask_pred(name: str, args, q, k):
+def mask_pred(name, args, q, k):
     """Boolean [len(q), len(k)] from the reference's Triton rule (mask.py:825, 911, 1010-1012,
-    1145-1148, 1301-1304)."""
+    1145-1148, 1301-1304).  For a user-written mask ``name`` is the test's own statement of the
+    predicate, a callable ``(q[:, None], k[None, :], args) -> bool array``."""
     q = np.asarray(q, dtype=np.int64)[:, None]
     k = np.asarray(k, dtype=np.int64)[None, :]
+    if callable(name):
+        return np.broadcast_to(np.asarray(name(q, k, args), dtype=bool), (q.shape[0], k.shape[1])).copy()
     if name == "FullChillMask":
         return np.ones((q.shape[0], k.shape[1]), dtype=bool)
     if name == "CausalChillMask":
