@@ -20,7 +20,7 @@ built-in masks use into a library of its own that serves mask id ``MASK_USER``:
         def mask(q, k, seq_len, args): ...
 
 ``hip_functor`` is the BODY of ``chill::Mask<CHILL_MASK_USER>``; alternatively ``hip_header`` names a
-complete header file.  The library is built once per (class name, source text) under
+complete header file.  The library is built once per (class name, functor text, kernel sources) under
 ``chill-attention_amd/lib/user/`` and loaded from there afterwards; building needs ``hipcc`` and
 ``make`` and takes about 15 s.  ``ChillMask.verify`` checks the numpy rules against the compiled
 functor, so a wrong functor does not go unnoticed.
@@ -68,8 +68,18 @@ def functor_source(cls) -> str:
     return _WRAPPER.format(cls=cls.__name__, body=cls.hip_functor)
 
 
+def _kernel_sources_digest() -> bytes:
+    h = hashlib.sha1()
+    for name in sorted(os.listdir(CSRC_DIR)):
+        if name.endswith((".h", ".hip", ".cpp")) or name == "Makefile":
+            with open(os.path.join(CSRC_DIR, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.digest()
+
+
 def _key(cls) -> str:
-    digest = hashlib.sha1(functor_source(cls).encode()).hexdigest()[:12]
+    """One library per (class, functor text, kernel sources): editing either builds a new one."""
+    digest = hashlib.sha1(functor_source(cls).encode() + _kernel_sources_digest()).hexdigest()[:12]
     return f"{cls.__name__}-{digest}"
 
 

@@ -111,6 +111,13 @@ def test_tile_table():
                     # one wave per 32 resident rows, or (dK/dV) a pair of waves per 32 rows
                     assert c["rows"] in (32 * c["waves"], 16 * c["waves"]) and c["streamed"] % 32 == 0
                     assert 0 < c["lds_bytes"] <= 160 * 1024
+    # rows the tile sweep put into the table (mask- and head-dim-specific)
+    causal, window = ca.CausalChillMask(), ca.SlidingWindowChillMask(128, 128)
+    assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 128
+    assert tile_config(causal, 64, torch.float16, _lib.PASS_FWD)["streamed"] == 128
+    assert tile_config(causal, 32, torch.float16, _lib.PASS_FWD)["streamed"] == 64
+    assert tile_config(window, 64, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 64
+    assert (tile_config(window, 64, torch.bfloat16, _lib.PASS_DQ)["waves"], tile_config(causal, 64, torch.bfloat16, _lib.PASS_DQ)["waves"]) == (4, 8)
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
     assert tq == 32 * waves and tk % 32 == 0
     (dq_q, dq_k, _), (dk_q, dk_k, _) = _get_default_config_bwd(128, torch.bfloat16)
@@ -130,3 +137,16 @@ def test_cpu_tensors_are_refused():
     q = torch.randn(1, 1, 16, 16)
     with pytest.raises((RuntimeError, NotImplementedError)):
         ca.chill_attention(q, q, q, mask=ca.CausalChillMask())
+
+
+def test_tile_sweep_candidates():
+    """The sweep tool's candidate list: the shipped shape comes first and overrides nothing."""
+    from chill_attention import tune
+
+    names = [n for n, _ in tune.CANDIDATES]
+    assert len(set(names)) == len(names) and tune.CANDIDATES[0][1] == {}
+    allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_DQ_WAVES", "CHILL_TUNE_DQ_STREAMED"}
+    header = open(os.path.join(ROOT, "chill-attention_amd", "csrc", "chill_tiles.h")).read()
+    for _, macros in tune.CANDIDATES:
+        assert set(macros) <= allowed and all(m in header for m in macros)
+    assert tune.candidate_library("w8_s64").endswith(os.path.join("lib", "tune", "w8_s64", "libchill_attention_hip.so"))
