@@ -213,6 +213,45 @@ def test_opcheck_and_compile():
     assert q.grad is not None and torch.isfinite(q.grad).all()
 
 
+@pytest.mark.parametrize("m", [MASK_INSTANCES[1], MASK_INSTANCES[2]], ids=mask_id)
+def test_hip_graph_replays(m):
+    """Forward + backward captured once in a HIP graph: every replay, with new contents in the
+    static inputs and eager work and synchronisations in between, equals the eager result.  (The
+    library allocates nothing, keeps no state and launches only on the caller's stream.)"""
+    mask = make_mask(m)
+    B, H, Hkv, T, D = 2, 4, 2, 300, 128
+    q, k, v = (torch.randn(B, h, T, D, device=DEV, dtype=torch.bfloat16, requires_grad=True) for h in (H, Hkv, Hkv))
+    do = torch.randn(B, H, T, D, device=DEV, dtype=torch.bfloat16)
+    lens = torch.tensor([T, 77], dtype=torch.int32, device=DEV)
+
+    def step():
+        out = ca.chill_attention(q, k, v, mask=mask, lens=lens)
+        grads = torch.autograd.grad(out, (q, k, v), do)
+        return (out,) + grads
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step()
+    for replay in range(4):
+        with torch.no_grad():
+            for t in (q, k, v, do):
+                t.copy_(torch.randn_like(t) * (1.0 + replay))
+            lens.copy_(torch.tensor([T - 13 * replay, 77 + 50 * replay], dtype=torch.int32))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in static_out]
+        want = step()
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w), f"replay {replay}"
+
+
 def test_device_functors_equal_host():
     """The mask functors and tile decisions as executed ON THE GPU equal the host build bit for bit."""
     import ctypes
