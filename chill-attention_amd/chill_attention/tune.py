@@ -36,6 +36,9 @@ CANDIDATES = [
     ("w4_s64", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4}),
     ("w4_s32", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4,
                 "CHILL_TUNE_FWD_STREAMED": 32, "CHILL_TUNE_DQ_STREAMED": 32}),
+    # dK/dV with 64 key rows per wave, K in registers and the accumulators in hand-managed accumulation
+    # registers (head dims 64 and 128): as fast as the shipped paired kernel, not faster
+    ("dkdv_r64", {"CHILL_TUNE_DKDV_R64": 1, "__flags__": "-mllvm -amdgpu-spill-vgpr-to-agpr=0"}),
 ]
 
 _HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Wno-unused-value",
@@ -48,7 +51,8 @@ def candidate_library(name: str) -> str:
 
 def build_candidates(jobs: int = 8) -> None:
     for name, macros in CANDIDATES:
-        extra = " ".join(f"-D{k}={v}" for k, v in macros.items())
+        extra = " ".join(f"-D{k}={v}" for k, v in macros.items() if k != "__flags__")
+        extra = (extra + " " + macros.get("__flags__", "")).strip()
         cmd = ["make", "-C", CSRC_DIR, f"-j{jobs}", f"EXTRA={extra}",
                f"BUILD={os.path.join(TUNE_BUILD_DIR, name)}", f"LIBDIR={os.path.dirname(candidate_library(name))}"]
         print("building", name, extra, flush=True)
@@ -64,7 +68,8 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
             out = os.path.join(tmp, unit + ".s")
             cmd = ["hipcc", *_HIPFLAGS, f"-I{os.path.join(_ROOT, '..', 'include')}",
                    f"-DCHILL_ELEM={elem}_t", f"-DCHILL_ELEM_NAME={elem}", f"-DCHILL_HEAD_DIM={dim}",
-                   *[f"-D{k}={v}" for k, v in (macros or {}).items()],
+                   *[f"-D{k}={v}" for k, v in (macros or {}).items() if k != "__flags__"],
+                   *(macros or {}).get("__flags__", "").split(),
                    "--cuda-device-only", "-S", os.path.join(CSRC_DIR, unit), "-o", out]
             subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
             text = open(out).read()

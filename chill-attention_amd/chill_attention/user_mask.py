@@ -108,6 +108,11 @@ def build(cls, force: bool = False, jobs: int = 8) -> str:
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0 or not os.path.exists(path):
         raise RuntimeError(f"{cls.__name__}: building the mask library failed:\n{res.stdout[-4000:]}")
+    # libraries of this class built from older sources (another key) are of no use any more
+    for root in (USER_BUILD_DIR, os.path.dirname(os.path.dirname(path))):
+        for name in os.listdir(root):
+            if name.startswith(cls.__name__ + "-") and name != _key(cls):
+                shutil.rmtree(os.path.join(root, name), ignore_errors=True)
     return path
 
 

@@ -1,0 +1,265 @@
+// dK/dV, register-resident variant for 16-bit rows of at most 256 bytes.
+//
+// A workgroup of 4 waves (one per SIMD, so each wave may use the whole 512-entry register file)
+// owns 256 key rows, 64 per wave.  A wave keeps its K rows in registers as MFMA B operands (the V
+// rows stay in LDS: both would not fit beside the score blocks) and its dK^T / dV^T accumulators
+// (2 key blocks x D/32 head-dim blocks x 16 registers each) in the accumulation registers under fixed
+// names (see the hand-placed MFMA helpers in chill_device.h).  Streamed through the LDS
+// ring: Q and dO tiles of 32 query rows with their LSE2 / delta, for every query head of the GQA
+// group in turn (chill_bwd_dkdv.py:156).
+//
+// Every streamed operand fetched from LDS feeds two MFMAs (one per 32-key block of the wave) and K
+// is never re-read: 0.75 KiB of LDS traffic per MFMA where the paired kernel needs 1.5 KiB.
+//
+// Built only with -DCHILL_TUNE_DKDV_R64=1, which needs -mllvm -amdgpu-spill-vgpr-to-agpr=0 next to it
+// (the accumulation registers are managed by hand).  Measured on the causal bf16 B8 H16 T8192 D128
+// workload it is as fast as the paired kernel (4.2-4.6 ms, box to box), not faster: with one wave per
+// SIMD the vector work hides only behind the wave's own MFMAs (0.9 ms of it stays exposed) and the
+// per-tile synchronisation costs as much again, so the table keeps the paired kernel.
+//
+//   S = Q K^T, dP = dO V^T, P = exp2(S * scale - LSE2), dS = P o (dP - delta),
+//   dV^T += dO^T P, dK^T += Q^T dS, finally dK *= sm_scale            (chill_bwd_dkdv.py:362-403, 230)
+#pragma once
+
+#include "chill_device.h"
+#include "chill_params.h"
+#include "chill_tiles.h"
+
+namespace chill {
+
+template <typename E, int D, int MASK, int NS>
+__global__ __launch_bounds__(256) void dkdv_r64_kernel(BwdParams p, int n_k_tiles, int total_items,
+                                                       int wave_has_full_blocks) {
+    using ET = typename Elem<E>::type;
+    static_assert(Elem<E>::k16, "16-bit element types");
+    typedef LdsTile<E, D> L;
+    constexpr int NW = 4;
+    constexpr int NT = NW * 64;
+    constexpr int KPW = 64;          // key rows per wave: two 32-key blocks
+    constexpr int TKR = NW * KPW;    // key rows per workgroup
+    constexpr int TQS = 32;          // streamed query rows per tile
+    constexpr int DB = (D + 31) / 32;
+    constexpr int NJ = Resident<E, D>::NJ;
+    constexpr int TILE_BYTES = L::bytes(TQS);
+    constexpr int VEC_BYTES = TQS * 4;
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * VEC_BYTES;  // Q, dO, LSE2, delta
+    constexpr int V_BYTES = L::bytes(TKR);                       // the workgroup's V rows, then the ring
+    constexpr int LA = NS - 2;  // tiles resident ahead of the one being consumed
+    static_assert(NS >= 2 && NS <= 4, "ring stages");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    if (item < 0) return;
+    const int bh = item / n_k_tiles;
+    // key tiles first-to-last: for causal-like masks the longest run first
+    const int ktile = item % n_k_tiles;
+    const int b = bh / p.H_kv;
+    const int hkv = bh % p.H_kv;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 31;
+    const int h = lane >> 5;
+
+    int seq_len = p.T;
+    if (p.lens != nullptr) seq_len = imin(p.lens[(int64_t)b * p.lens_stride], p.T);
+
+    const int kb0 = ktile * TKR;
+    ET* dkbase = reinterpret_cast<ET*>(p.dk) + b * p.sdk.b + hkv * p.sdk.h;
+    ET* dvbase = reinterpret_cast<ET*>(p.dv) + b * p.sdv.b + hkv * p.sdv.h;
+    if (kb0 >= seq_len) {
+        int nrows = imin(TKR, p.T - kb0);
+        zero_rows<E, D, NT>(dkbase, p.sdk.t, kb0, nrows, tid);
+        zero_rows<E, D, NT>(dvbase, p.sdv.t, kb0, nrows, tid);
+        return;
+    }
+
+    const TileRange wg = tile_range<MASK, false>(kb0, TKR, TQS, seq_len, false, p.margs);
+    const int n_tiles = wg.end - wg.start;
+    const int n_iters = n_tiles * p.group;
+
+    AsyncSwizzledLoader<E, D, TQS, NT> load_q, load_do;
+    load_q.init(p.sq.t, wave, lane);
+    load_do.init(p.sdo.t, wave, lane);
+    // iteration it = (group head g, q-tile): stage it % NS
+    auto issue_iter = [&](int it, int st_index) {
+        const int g = it / n_tiles;
+        const int q0 = (wg.start + it % n_tiles) * TQS;
+        const int hq = hkv * p.group + g;
+        char* st = smem + V_BYTES + st_index * STAGE_BYTES;
+        const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
+        const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
+        load_q.issue(qptr + (int64_t)q0 * p.sq.t, p.T - q0, st, wave, lane);
+        load_do.issue(doptr + (int64_t)q0 * p.sdo.t, p.T - q0, st + TILE_BYTES, wave, lane);
+        if (wave == NW - 1 && lane < TQS) {
+            // LSE2 and delta of the tile's rows; rows past the end of the tensor read as zero
+            const float* lse = p.lse + b * p.lse_b + hq * p.lse_h + q0;
+            const float* del = p.delta + b * p.delta_b + hq * p.delta_h + q0;
+            char* vec = st + 2 * TILE_BYTES;
+            if (q0 + lane < p.T) {
+                async_load4(lse, lane * 4, lds_address(vec));
+                async_load4(del, lane * 4, lds_address(vec + VEC_BYTES));
+            } else {
+                reinterpret_cast<float*>(vec)[lane] = 0.f;
+                reinterpret_cast<float*>(vec + VEC_BYTES)[lane] = 0.f;
+            }
+        }
+    };
+    {
+        AsyncSwizzledLoader<E, D, TKR, NT> load_v;
+        const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
+        load_v.init(p.sv.t, wave, lane);
+        load_v.issue(vptr + (int64_t)kb0 * p.sv.t, p.T - kb0, smem, wave, lane);
+    }
+#pragma unroll
+    for (int i = 0; i <= LA; i++)
+        if (i < n_iters) issue_iter(i, i);
+
+    const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
+    const int kw = kb0 + KPW * wave;
+    OperandOffsets<E, D> ofs;
+    ofs.init(lane);
+    Resident<E, D> kf[2];
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+        load_resident<E, D>(kf[c], kptr + (int64_t)(kw + 32 * c) * p.sk.t, p.sk.t, p.T - kw - 32 * c, lane);
+
+    TileRange wr = {wg.start, wg.start, wg.start, wg.start};
+    if (kw < seq_len) wr = tile_range<MASK, false>(kw, KPW, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
+    const int ta = wr.start - wg.start, tb = wr.end - wg.start;
+    const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
+
+    // accumulation registers: dV^T block (c, db) at a[16 * (c * DB + db)], dK^T blocks after them
+    constexpr int DV_BASE = 0, DK_BASE = 2 * DB * 16;
+    agpr_reserve();
+    int tok = agpr_zero<0, 4 * DB * 16>();
+    const float scale = p.scale_log2;
+    const float masked_score = scale < 0.f ? INFINITY : -INFINITY;  // times the scale: -inf
+    const lds_char* lds0 = (const lds_char*)smem;
+    // the resident operands must have arrived before the loop, where the only vector-memory traffic
+    // is the async tile loads and no compiler-placed wait may cover them
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(kf[c].c[j]));
+
+    int st_cur = NS - 1;
+    int st_issue = LA;
+    int tile = -1;  // position of iteration `it` inside the q-tile range (it % n_tiles)
+    for (int it = 0; it < n_iters; it++) {
+        wait_async_tiles();
+        __syncthreads();
+        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        tile = tile + 1 == n_tiles ? 0 : tile + 1;
+        if (it + LA + 1 < n_iters) issue_iter(it + LA + 1, st_issue);
+        if (tile < ta || tile >= tb) continue;
+        const lds_char* q_tile = lds0 + V_BYTES + st_cur * STAGE_BYTES;
+        const lds_char* do_tile = q_tile + TILE_BYTES;
+        const lds_float* vec = reinterpret_cast<const lds_float*>(q_tile + 2 * TILE_BYTES);
+        const bool full = (tile >= fa) && (tile < fb);
+        const int q0 = (wg.start + tile) * TQS;
+
+        f32x4 lse4[4], del4[4];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++)
+            lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
+        f32x16 s[2], dp[2];
+        // S = Q K^T: one Q chunk from LDS feeds both key blocks
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const i32x4 a = ofs.row_chunk(q_tile, 0, j, lane);
+            if (j == 0) {
+                Mfma16<E>::set(a, kf[0].c[j], s[0], tok);
+                Mfma16<E>::set(a, kf[1].c[j], s[1], tok);
+            } else {
+                Mfma16<E>::add(a, kf[0].c[j], s[0], tok);
+                Mfma16<E>::add(a, kf[1].c[j], s[1], tok);
+            }
+        }
+        // dP = dO V^T
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const i32x4 a = ofs.row_chunk(do_tile, 0, j, lane);
+            const i32x4 v0 = ofs.row_chunk(lds0, 2 * wave, j, lane);
+            const i32x4 v1 = ofs.row_chunk(lds0, 2 * wave + 1, j, lane);
+            if (j == 0) {
+                Mfma16<E>::set(a, v0, dp[0], tok);
+                Mfma16<E>::set(a, v1, dp[1], tok);
+            } else {
+                Mfma16<E>::add(a, v0, dp[0], tok);
+                Mfma16<E>::add(a, v1, dp[1], tok);
+            }
+        }
+        mfma_fence(s[0], s[1], dp[0], dp[1]);
+        if (!full) {
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const int k_pos = kw + 32 * c + n;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
+                    const bool ok = (q < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(q, k_pos, seq_len, p.margs);
+                    s[c][r] = ok ? s[c][r] : masked_score;
+                }
+            }
+            // a row that attends to nothing has LSE2 = -inf and only masked entries
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float l = lse4[r / 4][r % 4];
+                lse4[r / 4][r % 4] = (l == -INFINITY) ? 0.f : l;
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[c][r] = fast_exp2(__builtin_fmaf(s[c][r], scale, -lse4[r / 4][r % 4]));
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++)
+            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
+        // dV^T += dO^T P: one transposed dO operand feeds both key blocks
+        {
+            i32x4 pb[2][2];
+            pack_block<E>(s[0], pb[0]);
+            pack_block<E>(s[1], pb[1]);
+            static_for<2>([&](auto sx) {
+                static_for<DB>([&](auto db) {
+                    const i32x4 a = ofs.tr_operand(do_tile, 0, sx, db, lane);
+                    Mfma16<E>::template acc<DV_BASE + 16 * db>(a, pb[0][sx], tok);
+                    Mfma16<E>::template acc<DV_BASE + 16 * (DB + db)>(a, pb[1][sx], tok);
+                });
+            });
+        }
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) dp[c][r] = s[c][r] * (dp[c][r] - del4[r / 4][r % 4]);
+        // dK^T += Q^T dS
+        {
+            i32x4 sb[2][2];
+            pack_block<E>(dp[0], sb[0]);
+            pack_block<E>(dp[1], sb[1]);
+            static_for<2>([&](auto sx) {
+                static_for<DB>([&](auto db) {
+                    const i32x4 a = ofs.tr_operand(q_tile, 0, sx, db, lane);
+                    Mfma16<E>::template acc<DK_BASE + 16 * db>(a, sb[0][sx], tok);
+                    Mfma16<E>::template acc<DK_BASE + 16 * (DB + db)>(a, sb[1][sx], tok);
+                });
+            });
+        }
+    }
+
+    agpr_drain(tok);
+    static_for<2>([&](auto c) {
+        const int k_pos = kw + 32 * c + n;
+        f32x16 acc[DB];
+        const bool valid = k_pos < seq_len;
+        static_for<DB>([&](auto db) { acc[db] = agpr_read_block<DK_BASE + 16 * (c * DB + db)>(); });
+        if (k_pos < p.T) store_row_transposed<E, D>(dkbase + (int64_t)k_pos * p.sdk.t, acc, p.sm_scale, valid, h);
+        static_for<DB>([&](auto db) { acc[db] = agpr_read_block<DV_BASE + 16 * (c * DB + db)>(); });
+        if (k_pos < p.T) store_row_transposed<E, D>(dvbase + (int64_t)k_pos * p.sdv.t, acc, 1.f, valid, h);
+    });
+}
+
+}  // namespace chill

@@ -18,6 +18,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <utility>
+
 #include "chill_mask.h"
 
 namespace chill {
@@ -122,6 +124,111 @@ __device__ __forceinline__ float sum_across_halves(float x) {
     int xi = __builtin_bit_cast(int, x);
     auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
     return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+}
+
+// ------------------------------------------------------------------------------------------
+// Hand-placed MFMAs (16-bit types).  A kernel that runs one wave per SIMD owns 512 registers per
+// lane: 256 ordinary ones, which the compiler allocates, and the 256 accumulation registers
+// a0..a255, which such a kernel manages by itself: blocks that only MFMAs touch for a whole loop
+// live there under fixed names, out of the compiler's sight (given the choice, the compiler moves a
+// block between the two files around every use).  Rules for a kernel that uses these helpers:
+//   * it calls agpr_reserve() first (declares a0..a255 used, so the wave gets all 512 registers)
+//     and is built with -mllvm -amdgpu-spill-vgpr-to-agpr=0, so the compiler never puts
+//     anything of its own there;
+//   * it contains no MFMA builtin (their results would be routed through the same registers);
+//   * the compiler does not see the latency of these instructions: mfma_fence() stands between
+//     the last MFMA that writes a block of ordinary registers and the first other instruction that
+//     reads it, agpr_drain() between the last accumulating MFMA and agpr_read_block().
+// All of them are volatile asm statements: they keep their program order.
+// ------------------------------------------------------------------------------------------
+#define CHILL_A10(b) "a" #b "0", "a" #b "1", "a" #b "2", "a" #b "3", "a" #b "4", "a" #b "5", "a" #b "6", "a" #b "7", "a" #b "8", "a" #b "9"
+__device__ __forceinline__ void agpr_reserve() {
+    asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", CHILL_A10(1), CHILL_A10(2), CHILL_A10(3),
+                 CHILL_A10(4), CHILL_A10(5), CHILL_A10(6), CHILL_A10(7), CHILL_A10(8), CHILL_A10(9), CHILL_A10(10),
+                 CHILL_A10(11), CHILL_A10(12), CHILL_A10(13), CHILL_A10(14), CHILL_A10(15), CHILL_A10(16), CHILL_A10(17),
+                 CHILL_A10(18), CHILL_A10(19), CHILL_A10(20), CHILL_A10(21), CHILL_A10(22), CHILL_A10(23), CHILL_A10(24),
+                 "a250", "a251", "a252", "a253", "a254", "a255");
+}
+#undef CHILL_A10
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{})
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+template <int I>
+__device__ __forceinline__ void agpr_zero_one() {
+    asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(I));
+}
+template <int BASE, int... I>
+__device__ __forceinline__ void agpr_zero_seq(std::integer_sequence<int, I...>) {
+    (agpr_zero_one<BASE + I>(), ...);
+}
+// a[BASE .. BASE + N - 1] = 0; returns the token the accumulating MFMAs are chained on
+template <int BASE, int N>
+__device__ __forceinline__ int agpr_zero() {
+    agpr_zero_seq<BASE>(std::make_integer_sequence<int, N>{});
+    int tok;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(tok));
+    return tok;
+}
+
+template <int I>
+__device__ __forceinline__ float agpr_read_one() {
+    float x;
+    asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(x) : "n"(I));
+    return x;
+}
+template <int BASE, int... I>
+__device__ __forceinline__ f32x16 agpr_read_seq(std::integer_sequence<int, I...>) {
+    f32x16 r;
+    ((r[I] = agpr_read_one<BASE + I>()), ...);
+    return r;
+}
+// the 32x32 accumulator block held in a[BASE .. BASE + 15]
+template <int BASE>
+__device__ __forceinline__ f32x16 agpr_read_block() {
+    return agpr_read_seq<BASE>(std::make_integer_sequence<int, 16>{});
+}
+__device__ __forceinline__ void agpr_drain(int tok) { asm volatile("s_nop 15\n\ts_nop 15" ::"v"(tok) : "memory"); }
+
+// `tok` threads a data dependency through the MFMAs: it keeps them in program order, and the
+// accumulating ones (which have no other output the compiler can see) alive, without making them
+// volatile (LDS reads may not move across a volatile asm statement, and each one would then expose its
+// full latency).  Program order matters: an MFMA that reads the block the MFMA just before it wrote
+// gives wrong results here, so the callers alternate between two blocks.  The chain starts at
+// agpr_zero() and ends in agpr_drain().
+template <typename E>
+struct Mfma16;
+#define CHILL_MFMA16(TYPE, MNEMONIC)                                                                          \
+    template <>                                                                                               \
+    struct Mfma16<TYPE> {                                                                                     \
+        /* a[BASE .. BASE+15] += A B; an operand written by the vector ALU just before needs the 2 wait states */ \
+        template <int BASE>                                                                                   \
+        __device__ __forceinline__ static void acc(i32x4 a, i32x4 b, int& tok) {                              \
+            asm("s_nop 1\n\t" MNEMONIC " a[%3:%4], %1, %2, a[%3:%4]"                                          \
+                : "+v"(tok) : "v"(a), "v"(b), "n"(BASE), "n"(BASE + 15));                                     \
+        }                                                                                                     \
+        /* c = A B and c += A B with c in ordinary registers */                                               \
+        __device__ __forceinline__ static void set(i32x4 a, i32x4 b, f32x16& c, int& tok) {                   \
+            asm(MNEMONIC " %0, %2, %3, 0" : "=&v"(c), "+v"(tok) : "v"(a), "v"(b));                            \
+        }                                                                                                     \
+        __device__ __forceinline__ static void add(i32x4 a, i32x4 b, f32x16& c, int& tok) {                   \
+            asm(MNEMONIC " %0, %2, %3, %0" : "+v"(c), "+v"(tok) : "v"(a), "v"(b));                            \
+        }                                                                                                     \
+    };
+CHILL_MFMA16(bf16_t, "v_mfma_f32_32x32x16_bf16")
+CHILL_MFMA16(f16_t, "v_mfma_f32_32x32x16_f16")
+#undef CHILL_MFMA16
+
+// An 8-pass MFMA needs 11 wait states before another kind of instruction may read its result.
+__device__ __forceinline__ void mfma_fence(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
+    asm volatile("s_nop 11" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -439,6 +546,19 @@ __device__ __forceinline__ f32x16 mma_rowwise(const lds_char* tile, int kb, cons
 #pragma unroll
     for (int j = 0; j < Resident<E, D>::NJ; j++) acc = Elem<E>::mma(ofs.row_chunk(tile, kb, j, lane), b.c[j], acc);
     return acc;
+}
+
+// The two 16-bit B operands a 32x32 accumulator-layout block packs into: operand s holds, for lane
+// (n, h), rows {16*s + 8*(e/4) + 4*h + e%4, e = 0..7} of column n.
+template <typename E>
+__device__ __forceinline__ void pack_block(const f32x16& p, i32x4 (&bop)[2]) {
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        f32x8 ps;
+#pragma unroll
+        for (int e = 0; e < 8; e++) ps[e] = p[8 * s + e];
+        bop[s] = Elem<E>::pack8(ps);
+    }
 }
 
 // acc(32 out-rows x 32 cols) += X^T * P: contraction over the 32 rows of block kb of the LDS tile,

@@ -25,6 +25,10 @@
 #define CHILL_TUNE_DQ_STREAMED 0
 #endif
 
+#ifndef CHILL_TUNE_DKDV_R64
+#define CHILL_TUNE_DKDV_R64 0
+#endif
+
 namespace chill {
 
 constexpr int elem_bytes(int dtype) { return dtype == CHILL_F32 ? 4 : 2; }
@@ -85,9 +89,18 @@ constexpr int dkdv_wide_stages(int streamed, int D, int dtype) {
     return 3 * dkdv_wide_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
 
+// Register-resident dK/dV kernel (16-bit, 128- or 256-byte rows): 4 waves x 64 key rows, K and V in
+// registers, 32-row Q / dO tiles in a ring of four stages.
+constexpr bool dkdv_is_r64(int D, int dtype) {
+    return CHILL_TUNE_DKDV_R64 && dtype != CHILL_F32 && (D == 64 || D == 128);
+}
+constexpr int kDkdvR64Stages = 4;
+
 constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
     const int row_bytes = D * elem_bytes(dtype);
+    if (dkdv_is_r64(D, dtype))
+        return TileConfig{256, 32, 4, 256 * row_bytes + kDkdvR64Stages * (2 * 32 * row_bytes + 2 * 32 * 4)};
     if (dkdv_is_paired(D, dtype))
         return TileConfig{128, 64, 8, 2 * 128 * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4)};
     return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};

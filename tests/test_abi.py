@@ -145,8 +145,9 @@ def test_tile_sweep_candidates():
 
     names = [n for n, _ in tune.CANDIDATES]
     assert len(set(names)) == len(names) and tune.CANDIDATES[0][1] == {}
-    allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_DQ_WAVES", "CHILL_TUNE_DQ_STREAMED"}
+    allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_DQ_WAVES", "CHILL_TUNE_DQ_STREAMED",
+               "CHILL_TUNE_DKDV_R64", "__flags__"}
     header = open(os.path.join(ROOT, "chill-attention_amd", "csrc", "chill_tiles.h")).read()
     for _, macros in tune.CANDIDATES:
-        assert set(macros) <= allowed and all(m in header for m in macros)
+        assert set(macros) <= allowed and all(m in header for m in macros if m != "__flags__")
     assert tune.candidate_library("w8_s64").endswith(os.path.join("lib", "tune", "w8_s64", "libchill_attention_hip.so"))
