@@ -326,18 +326,20 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
 // pair add up to the same amount for every workgroup and the grid finishes without a tail.
 template <typename E, int D, int MASK, int NW, int TK, int NS>
 __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
-                                                      int wave_has_full_blocks) {
+                                                      int wave_has_full_blocks, int paired) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
     if (item < 0) return;
-    const int n_pairs = (n_q_tiles + 1) / 2;
-    const int bh = item / n_pairs;
-    const int j = item % n_pairs;
+    // paired: a workgroup takes q-tile j from the end and q-tile j from the start (equal work under
+    // causal-like masks); unpaired: one q-tile per workgroup, last tiles first
+    const int per_head = paired ? (n_q_tiles + 1) / 2 : n_q_tiles;
+    const int bh = item / per_head;
+    const int j = item % per_head;
     const int b = bh / p.H;
     const int hd = bh % p.H;
     const int qt_hi = n_q_tiles - 1 - j;
     fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, wave_has_full_blocks);
-    if (j != qt_hi) {
+    if (paired && j != qt_hi) {
         __syncthreads();  // the LDS ring is reused
         fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
     }
@@ -345,6 +347,10 @@ __global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles
 
 // Launcher for one (element type, head dim); dispatches on the mask id and takes the tile shape
 // from the static table.
+// fewer paired workgroups than an MI355X has CUs: launch one q-tile per workgroup (measured on causal
+// shapes: 16-35 % faster below the threshold, 7-16 % slower at two to four times it)
+constexpr int kPairedMinWorkgroups = 256;
+
 template <typename E, int D>
 int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
     // the async loader keeps per-lane global offsets in 32 bits
@@ -358,7 +364,10 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES,
                       "table and kernel disagree on LDS");
         const int n_q_tiles = cdiv(p.T, cfg.rows);
-        const int64_t total64 = (int64_t)p.B * p.H * ((n_q_tiles + 1) / 2);
+        // pairing q-tiles balances long causal runs; with few workgroups it only halves the number of
+        // CUs that get work
+        const bool paired = (int64_t)p.B * p.H * ((n_q_tiles + 1) / 2) >= kPairedMinWorkgroups;
+        const int64_t total64 = (int64_t)p.B * p.H * (paired ? (n_q_tiles + 1) / 2 : n_q_tiles);
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
@@ -369,7 +378,7 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
                                     hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)
                 return CHILL_ERR_HIP;
         }
-        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
+        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0, paired ? 1 : 0);
         status = (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
     });
     return status;
