@@ -52,8 +52,7 @@ def candidate_library(name: str) -> str:
 def build_candidates(jobs: int = 8) -> None:
     for name, macros in CANDIDATES:
         extra = " ".join(f"-D{k}={v}" for k, v in macros.items() if k != "__flags__")
-        extra = (extra + " " + macros.get("__flags__", "")).strip()
-        cmd = ["make", "-C", CSRC_DIR, f"-j{jobs}", f"EXTRA={extra}",
+        cmd = ["make", "-C", CSRC_DIR, f"-j{jobs}", f"EXTRA={extra}", f"HIPEXTRA={macros.get('__flags__', '')}",
                f"BUILD={os.path.join(TUNE_BUILD_DIR, name)}", f"LIBDIR={os.path.dirname(candidate_library(name))}"]
         print("building", name, extra, flush=True)
         subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL)
