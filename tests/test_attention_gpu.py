@@ -252,6 +252,30 @@ def test_hip_graph_replays(m):
             assert torch.equal(g, w), f"replay {replay}"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("D", [16, 64, 128, 256])
+def test_delta_kernel(D, dtype):
+    """chill_bwd_delta through the C ABI against the closed form rowsum(O * dO) in fp64 (utils.py:190),
+    on strided inputs and a T that is not a multiple of the kernel's rows per block."""
+    import ctypes
+
+    from chill_attention import _lib
+
+    B, H, T = 3, 5, 333
+    o = torch.randn(B, T, H, D, device=DEV, dtype=dtype).transpose(1, 2)  # [B, H, T, D] view, strided
+    do = torch.randn(B, H, T, D, device=DEV, dtype=dtype)
+    delta = torch.full((B, H, T), float("nan"), device=DEV, dtype=torch.float32)
+    to, tdo = _lib.tensor4(o), _lib.tensor4(do)
+    _lib.check("chill_bwd_delta", _lib.lib.chill_bwd_delta(
+        ctypes.byref(to), ctypes.byref(tdo), ctypes.c_void_p(delta.data_ptr()), _lib.strides3(delta),
+        B, H, T, D, {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}[dtype],
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    want = orc.delta(o.double().cpu().numpy(), do.double().cpu().numpy())
+    # fp32 accumulation of D products of magnitude ~1
+    np.testing.assert_allclose(delta.cpu().numpy(), want, atol=2e-5 * D, rtol=1e-5)
+
+
 def test_device_functors_equal_host():
     """The mask functors and tile decisions as executed ON THE GPU equal the host build bit for bit."""
     import ctypes
