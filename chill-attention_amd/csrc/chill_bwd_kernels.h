@@ -175,6 +175,8 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
         lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
         delta_q = p.delta[b * p.delta_b + hd * p.delta_h + q_pos];
     }
+    // a row that attends to nothing has LSE2 = -inf and only masked entries (score -inf): P = exp2(-inf - 0)
+    if (lse_q == -INFINITY) lse_q = 0.f;
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
@@ -187,6 +189,7 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
 #pragma unroll
         for (int r = 0; r < 16; r++) dq[i][r] = 0.f;
     const float scale = p.scale_log2;
+    const float masked_score = scale < 0.f ? INFINITY : -INFINITY;  // times the scale: -inf
 
     // S^T = K Q^T and dP^T = V dO^T of step kb of the stage at `stage`
     auto gemms = [&](f32x16& sdst, f32x16& dpdst, const lds_char* stage, int kb) {
@@ -218,20 +221,26 @@ __global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles,
         const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
         const bool full = (i >= fa) && (i < fb);
         const int k0 = (wg.start + i) * TK;
+        // Masked entries get a score of -inf (times the sign of the scale) in a branch of their own, so that
+        // the rest of the tile is the same straight-line code for full and partial tiles, in which the
+        // compiler places the vector work of one 32-key step among the MFMAs of the next.
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
             f32x16 cs, cdp;
             gemms(cs, cdp, stage, kb);
-            auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
-                q = q_pos;
-                k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
-                lse = lse_q;
-                delta = delta_q;
-            };
-            if (full)
-                softmax_grad_block<MASK, false>(cs, cdp, scale, seq_len, p.margs, pos);
-            else
-                softmax_grad_block<MASK, true>(cs, cdp, scale, seq_len, p.margs, pos);
+            if (!full) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+                    const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
+                    cs[r] = ok ? cs[r] : masked_score;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float pv = fast_exp2(__builtin_fmaf(cs[r], scale, -lse_q));
+                cdp[r] = pv * (cdp[r] - delta_q);
+            }
             // dQ^T += K^T dS^T
             mma_transposed<E, D>(stage, kb, ofs, cdp, dq, lane);
         }
