@@ -221,8 +221,10 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
-    k_ms = [sum(ev[s][i][0].elapsed_time(ev[s][i][1]) for s in range(args.steps)) / args.steps
-            for i in range(len(kernels))]
+    per_launch = [[ev[s][i][0].elapsed_time(ev[s][i][1]) for s in range(args.steps)] for i in range(len(kernels))]
+    k_ms = [sum(x) / len(x) for x in per_launch]
+    k_min = [min(x) for x in per_launch]
+    k_med = [sorted(x)[len(x) // 2] for x in per_launch]
 
     nnz = mask.nnz(T)
     fwd_flops = 4.0 * B * H * D * nnz
@@ -273,6 +275,8 @@ def main():
                                f"sigma={sigma}, inputs resident in HBM"},
         "frac_of_peak": value / peak,
         "kernel_ms": {kernels[i][0]: k_ms[i] for i in range(len(kernels))},
+        "kernel_ms_median": {kernels[i][0]: k_med[i] for i in range(len(kernels))},
+        "kernel_ms_min": {kernels[i][0]: k_min[i] for i in range(len(kernels))},
         "fwd_tflops": fwd_flops / (k_ms[0] * 1e-3) / 1e12,
         "fwd_frac_of_peak": fwd_flops / (k_ms[0] * 1e-3) / 1e12 / peak,
         "roofline": roof,
