@@ -86,6 +86,55 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
     return rows
 
 
+def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | None = None) -> list:
+    """Kernels that name accumulation registers themselves (dkdv_regs_kernel) rely on the compiler
+    keeping out of them.  Compiles the backward translation unit of (elem, dim) to assembly and
+    returns, per such kernel, (name, highest accumulation register the COMPILER uses or -1, lowest one
+    the kernel's own asm statements name, spilled registers): sound iff the first is below the second
+    and nothing is spilled."""
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "bwd.s")
+        cmd = ["hipcc", *_HIPFLAGS, f"-I{os.path.join(_ROOT, '..', 'include')}",
+               f"-DCHILL_ELEM={elem}_t", f"-DCHILL_ELEM_NAME={elem}", f"-DCHILL_HEAD_DIM={dim}",
+               *[f"-D{k}={v}" for k, v in (macros or {}).items() if k != "__flags__"],
+               *(macros or {}).get("__flags__", "").split(),
+               "--cuda-device-only", "-S", os.path.join(CSRC_DIR, "chill_bwd_inst.hip"), "-o", out]
+        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        text = open(out).read()
+    spills = {}
+    for block in re.findall(r"- \.agpr_count:.*?\.wavefront_size:", text, flags=re.S):
+        name = re.search(r"\.name:\s+(\S+)", block).group(1)
+        spills[name] = int(re.search(r"\.vgpr_spill_count:\s+(\d+)", block).group(1))
+    rows, cur, in_asm = {}, None, False
+    for line in text.splitlines():
+        m = re.match(r"^(_ZN5chill\w+):", line)
+        if m:
+            cur = m.group(1) if "dkdv_regs_kernel" in m.group(1) else None
+            if cur:
+                rows[cur] = {"compiler": -1, "hand": 1 << 30}
+            continue
+        if line.startswith(".Lfunc_end"):
+            cur = None
+        if cur is None:
+            continue
+        if "#ASMSTART" in line:
+            in_asm = True
+            continue
+        if "#ASMEND" in line:
+            in_asm = False
+            continue
+        code = line.split(";")[0]
+        used = [int(x) for x in re.findall(r"\ba(\d+)\b", code)]
+        for lo, hi in re.findall(r"\ba\[(0x[0-9a-f]+|\d+)(?::(0x[0-9a-f]+|\d+))?\]", code):
+            used += [int(lo, 0), int(hi, 0) if hi else int(lo, 0)]
+        if used:
+            if in_asm:
+                rows[cur]["hand"] = min(rows[cur]["hand"], min(used))
+            else:
+                rows[cur]["compiler"] = max(rows[cur]["compiler"], max(used))
+    return [(k, v["compiler"], v["hand"], spills.get(k, -1)) for k, v in rows.items()]
+
+
 def time_candidates(workloads) -> list:
     """Kernel times of every built candidate on the given bench workloads (needs the GPU).  Each
     candidate runs in a process of its own, because a process binds one build of the library."""

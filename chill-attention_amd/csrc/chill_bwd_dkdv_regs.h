@@ -1,24 +1,28 @@
-// dK/dV, register-resident variant for 16-bit rows of at most 256 bytes.
+// dK/dV with the accumulators in hand-managed accumulation registers (16-bit inputs).
 //
 // A workgroup of 4 waves (one per SIMD, so each wave may use the whole 512-entry register file)
-// owns 256 key rows, 64 per wave.  A wave keeps its K rows in registers as MFMA B operands (the V
-// rows stay in LDS: both would not fit beside the score blocks) and its dK^T / dV^T accumulators
-// (2 key blocks x D/32 head-dim blocks x 16 registers each) in the accumulation registers under fixed
-// names (see the hand-placed MFMA helpers in chill_device.h).  Streamed through the LDS
-// ring: Q and dO tiles of 32 query rows with their LSE2 / delta, for every query head of the GQA
-// group in turn (chill_bwd_dkdv.py:156).
-//
-// Every streamed operand fetched from LDS feeds two MFMAs (one per 32-key block of the wave) and K
-// is never re-read: 0.75 KiB of LDS traffic per MFMA where the paired kernel needs 1.5 KiB.
-//
-// Built only with -DCHILL_TUNE_DKDV_R64=1, which needs -mllvm -amdgpu-spill-vgpr-to-agpr=0 next to it
-// (the accumulation registers are managed by hand).  Measured on the causal bf16 B8 H16 T8192 D128
-// workload it is as fast as the paired kernel (4.2-4.6 ms, box to box), not faster: with one wave per
-// SIMD the vector work hides only behind the wave's own MFMAs (0.9 ms of it stays exposed) and the
-// per-tile synchronisation costs as much again, so the table keeps the paired kernel.
+// owns 4 * CB * 32 key rows, CB blocks of 32 per wave.  A wave keeps its K rows in registers as MFMA
+// B operands (the V rows stay in LDS: both would not fit beside the score blocks) and its dK^T / dV^T
+// accumulators (CB x D/32 blocks of 16 registers each) in the accumulation registers under fixed
+// names (see the hand-placed MFMA helpers in chill_device.h).  Streamed through the LDS ring: Q and
+// dO tiles of 32 query rows with their LSE2 / delta, for every query head of the GQA group in turn
+// (chill_bwd_dkdv.py:156).
 //
 //   S = Q K^T, dP = dO V^T, P = exp2(S * scale - LSE2), dS = P o (dP - delta),
 //   dV^T += dO^T P, dK^T += Q^T dS, finally dK *= sm_scale            (chill_bwd_dkdv.py:362-403, 230)
+//
+// CB = 1, D = 256 (512-byte rows) is the shipped dK/dV kernel of that shape: 2 x 8 accumulator blocks
+// are exactly the 256 accumulation registers, which the compiler cannot keep there by itself (its
+// version of this kernel spills 2400 registers to scratch and runs 40x slower).
+// CB = 2, D = 64 / 128 is a sweep candidate (-DCHILL_TUNE_DKDV_R64=1): every streamed operand fetched
+// from LDS feeds two MFMAs and K is never re-read, 0.75 KiB of LDS traffic per MFMA where the paired
+// kernel needs 1.5 KiB.  On the causal bf16 B8 H16 T8192 D128 workload it is as fast as the paired
+// kernel (4.2-4.6 ms, box to box), not faster: with one wave per SIMD the vector work hides only
+// behind the wave's own MFMAs (0.9 ms of it stays exposed) and the per-tile synchronisation costs
+// as much again, so the table keeps the paired kernel there.
+//
+// Every translation unit that instantiates this kernel is checked (tests/test_abi.py) for the
+// compiler keeping out of the accumulation registers the kernel names itself.
 #pragma once
 
 #include "chill_device.h"
@@ -27,15 +31,15 @@
 
 namespace chill {
 
-template <typename E, int D, int MASK, int NS>
-__global__ __launch_bounds__(256) void dkdv_r64_kernel(BwdParams p, int n_k_tiles, int total_items,
+template <typename E, int D, int MASK, int CB, int NS>
+__global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_tiles, int total_items,
                                                        int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     static_assert(Elem<E>::k16, "16-bit element types");
     typedef LdsTile<E, D> L;
     constexpr int NW = 4;
     constexpr int NT = NW * 64;
-    constexpr int KPW = 64;          // key rows per wave: two 32-key blocks
+    constexpr int KPW = 32 * CB;     // key rows per wave: CB 32-key blocks
     constexpr int TKR = NW * KPW;    // key rows per workgroup
     constexpr int TQS = 32;          // streamed query rows per tile
     constexpr int DB = (D + 31) / 32;
@@ -120,9 +124,9 @@ __global__ __launch_bounds__(256) void dkdv_r64_kernel(BwdParams p, int n_k_tile
     const int kw = kb0 + KPW * wave;
     OperandOffsets<E, D> ofs;
     ofs.init(lane);
-    Resident<E, D> kf[2];
+    Resident<E, D> kf[CB];
 #pragma unroll
-    for (int c = 0; c < 2; c++)
+    for (int c = 0; c < CB; c++)
         load_resident<E, D>(kf[c], kptr + (int64_t)(kw + 32 * c) * p.sk.t, p.sk.t, p.T - kw - 32 * c, lane);
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
@@ -131,16 +135,17 @@ __global__ __launch_bounds__(256) void dkdv_r64_kernel(BwdParams p, int n_k_tile
     const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
 
     // accumulation registers: dV^T block (c, db) at a[16 * (c * DB + db)], dK^T blocks after them
-    constexpr int DV_BASE = 0, DK_BASE = 2 * DB * 16;
+    constexpr int DV_BASE = 0, DK_BASE = CB * DB * 16;
+    static_assert(2 * CB * DB * 16 <= 256, "accumulators exceed the accumulation registers");
     agpr_reserve();
-    int tok = agpr_zero<0, 4 * DB * 16>();
+    int tok = agpr_zero<0, 2 * CB * DB * 16>();
     const float scale = p.scale_log2;
     const float masked_score = scale < 0.f ? INFINITY : -INFINITY;  // times the scale: -inf
     const lds_char* lds0 = (const lds_char*)smem;
     // the resident operands must have arrived before the loop, where the only vector-memory traffic
     // is the async tile loads and no compiler-placed wait may cover them
 #pragma unroll
-    for (int c = 0; c < 2; c++)
+    for (int c = 0; c < CB; c++)
 #pragma unroll
         for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(kf[c].c[j]));
 
@@ -165,37 +170,36 @@ __global__ __launch_bounds__(256) void dkdv_r64_kernel(BwdParams p, int n_k_tile
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++)
             lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
-        f32x16 s[2], dp[2];
-        // S = Q K^T: one Q chunk from LDS feeds both key blocks
+        f32x16 s[CB], dp[CB];
+        // S = Q K^T and dP = dO V^T, chunk by chunk: one Q (dO) chunk from LDS feeds all key blocks, and
+        // consecutive MFMAs never write the same block
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
-            const i32x4 a = ofs.row_chunk(q_tile, 0, j, lane);
-            if (j == 0) {
-                Mfma16<E>::set(a, kf[0].c[j], s[0], tok);
-                Mfma16<E>::set(a, kf[1].c[j], s[1], tok);
-            } else {
-                Mfma16<E>::add(a, kf[0].c[j], s[0], tok);
-                Mfma16<E>::add(a, kf[1].c[j], s[1], tok);
-            }
-        }
-        // dP = dO V^T
+            const i32x4 aq = ofs.row_chunk(q_tile, 0, j, lane);
+            const i32x4 ado = ofs.row_chunk(do_tile, 0, j, lane);
 #pragma unroll
-        for (int j = 0; j < NJ; j++) {
-            const i32x4 a = ofs.row_chunk(do_tile, 0, j, lane);
-            const i32x4 v0 = ofs.row_chunk(lds0, 2 * wave, j, lane);
-            const i32x4 v1 = ofs.row_chunk(lds0, 2 * wave + 1, j, lane);
-            if (j == 0) {
-                Mfma16<E>::set(a, v0, dp[0], tok);
-                Mfma16<E>::set(a, v1, dp[1], tok);
-            } else {
-                Mfma16<E>::add(a, v0, dp[0], tok);
-                Mfma16<E>::add(a, v1, dp[1], tok);
+            for (int c = 0; c < CB; c++) {
+                if (j == 0)
+                    Mfma16<E>::set(aq, kf[c].c[j], s[c], tok);
+                else
+                    Mfma16<E>::add(aq, kf[c].c[j], s[c], tok);
+            }
+#pragma unroll
+            for (int c = 0; c < CB; c++) {
+                const i32x4 vc = ofs.row_chunk(lds0, CB * wave + c, j, lane);
+                if (j == 0)
+                    Mfma16<E>::set(ado, vc, dp[c], tok);
+                else
+                    Mfma16<E>::add(ado, vc, dp[c], tok);
             }
         }
-        mfma_fence(s[0], s[1], dp[0], dp[1]);
+        if constexpr (CB == 2)
+            mfma_fence(s[0], s[1], dp[0], dp[1]);
+        else
+            mfma_fence(s[0], dp[0]);
         if (!full) {
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
+            for (int c = 0; c < CB; c++) {
                 const int k_pos = kw + 32 * c + n;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
@@ -212,46 +216,44 @@ __global__ __launch_bounds__(256) void dkdv_r64_kernel(BwdParams p, int n_k_tile
             }
         }
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+        for (int c = 0; c < CB; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) s[c][r] = fast_exp2(__builtin_fmaf(s[c][r], scale, -lse4[r / 4][r % 4]));
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++)
             del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
-        // dV^T += dO^T P: one transposed dO operand feeds both key blocks
+        // dV^T += dO^T P: one transposed dO operand feeds all key blocks
         {
-            i32x4 pb[2][2];
-            pack_block<E>(s[0], pb[0]);
-            pack_block<E>(s[1], pb[1]);
+            i32x4 pb[CB][2];
+#pragma unroll
+            for (int c = 0; c < CB; c++) pack_block<E>(s[c], pb[c]);
             static_for<2>([&](auto sx) {
                 static_for<DB>([&](auto db) {
                     const i32x4 a = ofs.tr_operand(do_tile, 0, sx, db, lane);
-                    Mfma16<E>::template acc<DV_BASE + 16 * db>(a, pb[0][sx], tok);
-                    Mfma16<E>::template acc<DV_BASE + 16 * (DB + db)>(a, pb[1][sx], tok);
+                    static_for<CB>([&](auto c) { Mfma16<E>::template acc<DV_BASE + 16 * (c * DB + db)>(a, pb[c][sx], tok); });
                 });
             });
         }
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+        for (int c = 0; c < CB; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) dp[c][r] = s[c][r] * (dp[c][r] - del4[r / 4][r % 4]);
         // dK^T += Q^T dS
         {
-            i32x4 sb[2][2];
-            pack_block<E>(dp[0], sb[0]);
-            pack_block<E>(dp[1], sb[1]);
+            i32x4 sb[CB][2];
+#pragma unroll
+            for (int c = 0; c < CB; c++) pack_block<E>(dp[c], sb[c]);
             static_for<2>([&](auto sx) {
                 static_for<DB>([&](auto db) {
                     const i32x4 a = ofs.tr_operand(q_tile, 0, sx, db, lane);
-                    Mfma16<E>::template acc<DK_BASE + 16 * db>(a, sb[0][sx], tok);
-                    Mfma16<E>::template acc<DK_BASE + 16 * (DB + db)>(a, sb[1][sx], tok);
+                    static_for<CB>([&](auto c) { Mfma16<E>::template acc<DK_BASE + 16 * (c * DB + db)>(a, sb[c][sx], tok); });
                 });
             });
         }
     }
 
     agpr_drain(tok);
-    static_for<2>([&](auto c) {
+    static_for<CB>([&](auto c) {
         const int k_pos = kw + 32 * c + n;
         f32x16 acc[DB];
         const bool valid = k_pos < seq_len;

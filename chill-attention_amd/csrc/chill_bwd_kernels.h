@@ -21,7 +21,7 @@
 #include "chill_device.h"
 #include "chill_params.h"
 #include "chill_tiles.h"
-#include "chill_bwd_dkdv_r64.h"
+#include "chill_bwd_dkdv_regs.h"
 
 namespace chill {
 
@@ -735,9 +735,9 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType);
-        constexpr bool r64 = dkdv_is_r64(D, Elem<E>::kDType);
-        constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType) && !r64;
-        static_assert(r64 ? (cfg.rows == 256 && cfg.streamed == 32 && cfg.waves == 4) : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64) : (cfg.rows == cfg.waves * 32),
+        constexpr int CB = dkdv_regs_blocks(D, Elem<E>::kDType);
+        constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType) && CB == 0;
+        static_assert(CB > 0 ? (cfg.rows == 128 * CB && cfg.streamed == 32 && cfg.waves == 4) : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64) : (cfg.rows == cfg.waves * 32),
                       "tile table and kernel shape disagree");
         const int n_k_tiles = cdiv(p.T, cfg.rows);
         const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
@@ -745,14 +745,14 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
         void (*kern)(BwdParams, int, int, int);
-        if constexpr (r64)
-            kern = dkdv_r64_kernel<E, D, MASK_ID, kDkdvR64Stages>;
+        if constexpr (CB > 0)
+            kern = dkdv_regs_kernel<E, D, MASK_ID, CB, dkdv_regs_stages(D)>;
         else if constexpr (paired)
             kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, 2>;
         else
             kern = dkdv_wide_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, dkdv_wide_stages(cfg.streamed, D, Elem<E>::kDType)>;
         // mask rule order is (q tile, k tile): the streamed tile is the q tile here
-        const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, r64 ? 64 : 32, p.T, p.margs);
+        const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, CB > 0 ? 32 * CB : 32, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)

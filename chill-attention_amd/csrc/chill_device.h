@@ -230,6 +230,9 @@ CHILL_MFMA16(f16_t, "v_mfma_f32_32x32x16_f16")
 __device__ __forceinline__ void mfma_fence(f32x16& x0, f32x16& x1, f32x16& x2, f32x16& x3) {
     asm volatile("s_nop 11" : "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3));
 }
+__device__ __forceinline__ void mfma_fence(f32x16& x0, f32x16& x1) {
+    asm volatile("s_nop 11" : "+v"(x0), "+v"(x1));
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 

@@ -89,18 +89,27 @@ constexpr int dkdv_wide_stages(int streamed, int D, int dtype) {
     return 3 * dkdv_wide_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
 
-// Register-resident dK/dV kernel (16-bit, 128- or 256-byte rows): 4 waves x 64 key rows, K and V in
-// registers, 32-row Q / dO tiles in a ring of four stages.
-constexpr bool dkdv_is_r64(int D, int dtype) {
-    return CHILL_TUNE_DKDV_R64 && dtype != CHILL_F32 && (D == 64 || D == 128);
+// dK/dV with hand-managed accumulation registers (dkdv_regs_kernel, 16-bit inputs): 4 waves, K in
+// registers, V in LDS, 32-row Q / dO tiles in a ring.  blocks = 32-key blocks per wave:
+//   * head dim 256: one block per wave (128 key rows per workgroup), two ring stages: the shipped
+//     kernel of that shape;
+//   * head dim 64 / 128 with -DCHILL_TUNE_DKDV_R64=1: two blocks per wave (256 key rows), four stages:
+//     a sweep candidate.
+constexpr int dkdv_regs_blocks(int D, int dtype) {
+    if (dtype == CHILL_F32) return 0;
+    if (D == 256) return 1;
+    if (CHILL_TUNE_DKDV_R64 && (D == 64 || D == 128)) return 2;
+    return 0;
 }
-constexpr int kDkdvR64Stages = 4;
+constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
 
 constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
     (void)mask_id;
     const int row_bytes = D * elem_bytes(dtype);
-    if (dkdv_is_r64(D, dtype))
-        return TileConfig{256, 32, 4, 256 * row_bytes + kDkdvR64Stages * (2 * 32 * row_bytes + 2 * 32 * 4)};
+    if (dkdv_regs_blocks(D, dtype) > 0) {
+        const int rows = 4 * 32 * dkdv_regs_blocks(D, dtype);
+        return TileConfig{rows, 32, 4, rows * row_bytes + dkdv_regs_stages(D) * (2 * 32 * row_bytes + 2 * 32 * 4)};
+    }
     if (dkdv_is_paired(D, dtype))
         return TileConfig{128, 64, 8, 2 * 128 * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4)};
     return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
