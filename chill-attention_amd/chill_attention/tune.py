@@ -87,20 +87,22 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
 
 
 def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | None = None) -> list:
-    """Kernels that name accumulation registers themselves (dkdv_regs_kernel) rely on the compiler
-    keeping out of them.  Compiles the backward translation unit of (elem, dim) to assembly and
+    """Kernels that name accumulation registers themselves (fwd_regs_kernel, dq_regs_kernel, dkdv_regs_kernel) rely on the compiler
+    keeping out of them.  Compiles the translation units of (elem, dim) to assembly and
     returns, per such kernel, (name, highest accumulation register the COMPILER uses or -1, lowest one
     the kernel's own asm statements name, spilled registers): sound iff the first is below the second
     and nothing is spilled."""
+    text = ""
     with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "bwd.s")
-        cmd = ["hipcc", *_HIPFLAGS, f"-I{os.path.join(_ROOT, '..', 'include')}",
-               f"-DCHILL_ELEM={elem}_t", f"-DCHILL_ELEM_NAME={elem}", f"-DCHILL_HEAD_DIM={dim}",
-               *[f"-D{k}={v}" for k, v in (macros or {}).items() if k != "__flags__"],
-               *(macros or {}).get("__flags__", "").split(),
-               "--cuda-device-only", "-S", os.path.join(CSRC_DIR, "chill_bwd_inst.hip"), "-o", out]
-        subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
-        text = open(out).read()
+        for unit in ("chill_fwd_inst.hip", "chill_bwd_inst.hip"):
+            out = os.path.join(tmp, unit + ".s")
+            cmd = ["hipcc", *_HIPFLAGS, f"-I{os.path.join(_ROOT, '..', 'include')}",
+                   f"-DCHILL_ELEM={elem}_t", f"-DCHILL_ELEM_NAME={elem}", f"-DCHILL_HEAD_DIM={dim}",
+                   *[f"-D{k}={v}" for k, v in (macros or {}).items() if k != "__flags__"],
+                   *(macros or {}).get("__flags__", "").split(),
+                   "--cuda-device-only", "-S", os.path.join(CSRC_DIR, unit), "-o", out]
+            subprocess.run(cmd, check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            text += open(out).read()
     spills = {}
     for block in re.findall(r"- \.agpr_count:.*?\.wavefront_size:", text, flags=re.S):
         name = re.search(r"\.name:\s+(\S+)", block).group(1)
@@ -109,7 +111,7 @@ def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | No
     for line in text.splitlines():
         m = re.match(r"^(_ZN5chill\w+):", line)
         if m:
-            cur = m.group(1) if "dkdv_regs_kernel" in m.group(1) else None
+            cur = m.group(1) if "_regs_kernel" in m.group(1) else None
             if cur:
                 rows[cur] = {"compiler": -1, "hand": 1 << 30}
             continue

@@ -108,7 +108,7 @@ def build(cls, force: bool = False, jobs: int = 8) -> str:
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0 or not os.path.exists(path):
         raise RuntimeError(f"{cls.__name__}: building the mask library failed:\n{res.stdout[-4000:]}")
-    # the head-dim-256 dK/dV kernel names accumulation registers itself: make sure the compiler kept
+    # the 16-bit head-dim-256 kernels name accumulation registers themselves: make sure the compiler kept
     # out of them with this functor inlined (see tune.hand_managed_registers)
     from . import tune
 
@@ -119,7 +119,7 @@ def build(cls, force: bool = False, jobs: int = 8) -> str:
                 os.remove(path)
                 raise RuntimeError(
                     f"{cls.__name__}: with this functor the compiler uses accumulation registers "
-                    f"(up to a{compiler_max}) that the head-dim-256 dK/dV kernel manages itself, or spills "
+                    f"(up to a{compiler_max}) that the head-dim-256 kernels manage themselves, or spills "
                     f"({spilled}); simplify the functor (kernel {name})")
     # libraries of this class built from older sources (another key) are of no use any more
     for root in (USER_BUILD_DIR, os.path.dirname(os.path.dirname(path))):

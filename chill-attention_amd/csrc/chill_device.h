@@ -132,14 +132,17 @@ __device__ __forceinline__ float sum_across_halves(float x) {
 // a0..a255, which such a kernel manages by itself: blocks that only MFMAs touch for a whole loop
 // live there under fixed names, out of the compiler's sight (given the choice, the compiler moves a
 // block between the two files around every use).  Rules for a kernel that uses these helpers:
-//   * it calls agpr_reserve() first (declares a0..a255 used, so the wave gets all 512 registers)
-//     and is built with -mllvm -amdgpu-spill-vgpr-to-agpr=0, so the compiler never puts
-//     anything of its own there;
+//   * it calls agpr_reserve() first (declares a0..a255 used, so the wave gets all 512 registers);
+//   * it names its blocks from a255 downwards: a compiler that runs out of ordinary registers parks
+//     values in the lowest accumulation registers.  Whether it stayed below the hand-named ones is
+//     checked on the assembly of every build that instantiates such a kernel
+//     (chill_attention/tune.py, hand_managed_registers);
 //   * it contains no MFMA builtin (their results would be routed through the same registers);
 //   * the compiler does not see the latency of these instructions: mfma_fence() stands between
 //     the last MFMA that writes a block of ordinary registers and the first other instruction that
 //     reads it, agpr_drain() between the last accumulating MFMA and agpr_read_block().
-// All of them are volatile asm statements: they keep their program order.
+// Fences, drains and register reads are volatile asm statements; the MFMAs keep their program order
+// through a token (below).
 // ------------------------------------------------------------------------------------------
 #define CHILL_A10(b) "a" #b "0", "a" #b "1", "a" #b "2", "a" #b "3", "a" #b "4", "a" #b "5", "a" #b "6", "a" #b "7", "a" #b "8", "a" #b "9"
 __device__ __forceinline__ void agpr_reserve() {
@@ -200,9 +203,9 @@ __device__ __forceinline__ void agpr_drain(int tok) { asm volatile("s_nop 15\n\t
 // `tok` threads a data dependency through the MFMAs: it keeps them in program order, and the
 // accumulating ones (which have no other output the compiler can see) alive, without making them
 // volatile (LDS reads may not move across a volatile asm statement, and each one would then expose its
-// full latency).  Program order matters: an MFMA that reads the block the MFMA just before it wrote
-// gives wrong results here, so the callers alternate between two blocks.  The chain starts at
-// agpr_zero() and ends in agpr_drain().
+// full latency).  A chain of MFMAs that accumulate into one block may be issued back to back (the
+// hardware forwards the block); callers that have two independent chains alternate between them all the
+// same.  The chain of tokens starts at agpr_zero() and ends in agpr_drain().
 template <typename E>
 struct Mfma16;
 #define CHILL_MFMA16(TYPE, MNEMONIC)                                                                          \
@@ -233,6 +236,7 @@ __device__ __forceinline__ void mfma_fence(f32x16& x0, f32x16& x1, f32x16& x2, f
 __device__ __forceinline__ void mfma_fence(f32x16& x0, f32x16& x1) {
     asm volatile("s_nop 11" : "+v"(x0), "+v"(x1));
 }
+__device__ __forceinline__ void mfma_fence(f32x16& x0) { asm volatile("s_nop 11" : "+v"(x0)); }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -375,6 +379,15 @@ struct AsyncSwizzledLoader {
 
 // All asynchronous tile loads issued so far by this wave have landed in LDS.
 __device__ __forceinline__ void wait_async_tiles() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// All but the N most recent vector-memory operations of this wave have completed (loads complete in
+// issue order).  For a ring that keeps tiles in flight beyond the one about to be consumed: N = the
+// number of loads the wave issued for those newer tiles, or less.
+template <int N>
+__device__ __forceinline__ void wait_async_tiles_except() {
+    static_assert(N >= 0 && N <= 63, "the counter has six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 
 // ------------------------------------------------------------------------------------------
 // Padded LDS tile: rows of D elements at a pitch of RB + PAD bytes.  Addresses are affine in

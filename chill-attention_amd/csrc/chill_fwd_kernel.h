@@ -321,6 +321,10 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
     }
 }
 
+}  // namespace chill
+#include "chill_fwd_regs.h"
+namespace chill {
+
 // One workgroup per (batch, head, PAIR of q-tiles): tile j from the end, then tile j from the
 // start.  For causal-like masks the work of a q-tile grows with its index, so the two halves of a
 // pair add up to the same amount for every workgroup and the grid finishes without a tail.
@@ -372,6 +376,7 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
         auto kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
+        if constexpr (fwd_uses_regs(D, Elem<E>::kDType)) kern = fwd_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
         const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

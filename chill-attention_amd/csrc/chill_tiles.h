@@ -25,6 +25,15 @@
 #define CHILL_TUNE_DQ_STREAMED 0
 #endif
 
+#ifndef CHILL_TUNE_D256_STREAMED
+#define CHILL_TUNE_D256_STREAMED 64
+#endif
+#ifndef CHILL_TUNE_FWD_REGS
+#define CHILL_TUNE_FWD_REGS 1
+#endif
+#ifndef CHILL_TUNE_DQ_REGS_KEYS
+#define CHILL_TUNE_DQ_REGS_KEYS 32
+#endif
 #ifndef CHILL_TUNE_DKDV_R64
 #define CHILL_TUNE_DKDV_R64 0
 #endif
@@ -51,11 +60,15 @@ constexpr int fwd_stages_for(int streamed, int D, int dtype) {
 // head dims 64 and 128 (half the barriers per key; measured -12 % at D = 64, -8 % on the chunkwise
 // configuration, equal on the causal one), except for the sliding window, whose narrow band pays
 // for every partially used tile: 64 keys.
+// 16-bit inputs at head dim 256: fwd_regs_kernel (O^T in hand-managed accumulation registers).
+constexpr bool fwd_uses_regs(int D, int dtype) { return CHILL_TUNE_FWD_REGS && dtype != CHILL_F32 && D == 256; }
+
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
     const int tuned_streamed = (D >= 64 && mask_id != CHILL_MASK_SLIDING_WINDOW) ? 128 : 64;
     const int waves = fast16 ? (CHILL_TUNE_FWD_WAVES ? CHILL_TUNE_FWD_WAVES : 8) : 4;
-    const int streamed = fast16 ? (CHILL_TUNE_FWD_STREAMED ? CHILL_TUNE_FWD_STREAMED : tuned_streamed) : 32;
+    const int wide16 = (dtype != CHILL_F32 && D == 256) ? CHILL_TUNE_D256_STREAMED : 32;
+    const int streamed = fast16 ? (CHILL_TUNE_FWD_STREAMED ? CHILL_TUNE_FWD_STREAMED : tuned_streamed) : wide16;
     return TileConfig{waves * 32, streamed, waves,
                       fwd_stages_for(streamed, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
 }
@@ -67,11 +80,16 @@ constexpr int dq_stages_for(int streamed, int D, int dtype) {
 
 // dQ.  16-bit inputs, head dim <= 128: 8 waves x 64 streamed keys; for the sliding window at head
 // dim <= 64, 4 waves x 32 keys (measured -17 %: a 128-row workgroup spans fewer unused tiles).
+// 16-bit inputs at head dim 256: dq_regs_kernel (hand-managed accumulation registers), 4 waves,
+// dq_regs_keys streamed keys per tile (0: the shape is served by dq_kernel).
+constexpr int dq_regs_keys(int D, int dtype) { return (dtype != CHILL_F32 && D == 256) ? CHILL_TUNE_DQ_REGS_KEYS : 0; }
+
 constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
     const bool fast16 = dtype != CHILL_F32 && D <= 128;
+    const int wide = dq_regs_keys(D, dtype) > 0 ? dq_regs_keys(D, dtype) : 32;
     const bool narrow = mask_id == CHILL_MASK_SLIDING_WINDOW && D <= 64;
     const int waves = fast16 ? (CHILL_TUNE_DQ_WAVES ? CHILL_TUNE_DQ_WAVES : (narrow ? 4 : 8)) : 4;
-    const int streamed = fast16 ? (CHILL_TUNE_DQ_STREAMED ? CHILL_TUNE_DQ_STREAMED : (narrow ? 32 : 64)) : 32;
+    const int streamed = fast16 ? (CHILL_TUNE_DQ_STREAMED ? CHILL_TUNE_DQ_STREAMED : (narrow ? 32 : 64)) : wide;
     return TileConfig{waves * 32, streamed, waves,
                       dq_stages_for(streamed, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
 }
