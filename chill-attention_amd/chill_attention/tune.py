@@ -10,7 +10,7 @@ with the table overridden (``CHILL_TUNE_*`` macros of ``csrc/chill_tiles.h``):
     python -m chill_attention.tune time [C3 C2 ...]      # time every built candidate on the GPU, print a table
 
 ``build`` and ``time`` are separate because compiling belongs on the CPU and timing on the GPU box.
-The shipped table is the row that wins on the headline workload (causal, bf16, D = 128).
+The shipped table takes, per mask class and head dim, the row that wins on the BASELINE workloads.
 """
 
 from __future__ import annotations
@@ -30,12 +30,21 @@ TUNE_BUILD_DIR = os.path.join(_ROOT, "build", "tune")
 
 # (name, {macro: value}): forward and dQ shapes for 16-bit inputs with head dim <= 128
 CANDIDATES = [
-    ("w8_s64", {}),  # the shipped table: 8 waves (256 rows), 64 streamed rows, 3 LDS stages
-    ("w8_s32", {"CHILL_TUNE_FWD_STREAMED": 32, "CHILL_TUNE_DQ_STREAMED": 32}),
-    ("w8_s128", {"CHILL_TUNE_FWD_STREAMED": 128, "CHILL_TUNE_DQ_STREAMED": 128}),
-    ("w4_s64", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4}),
-    ("w4_s32", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4,
-                "CHILL_TUNE_FWD_STREAMED": 32, "CHILL_TUNE_DQ_STREAMED": 32}),
+    ("shipped", {}),  # the table as it ships
+    ("w8_s64", {"CHILL_TUNE_FWD_WAVES": 8, "CHILL_TUNE_DQ_WAVES": 8, "CHILL_TUNE_FWD_STREAMED": 64,
+                "CHILL_TUNE_DQ_STREAMED": 64, "CHILL_TUNE_FWD_STAGES": 3, "CHILL_TUNE_DQ_STAGES": 3}),
+    ("w8_s32", {"CHILL_TUNE_FWD_WAVES": 8, "CHILL_TUNE_DQ_WAVES": 8, "CHILL_TUNE_FWD_STREAMED": 32,
+                "CHILL_TUNE_DQ_STREAMED": 32, "CHILL_TUNE_FWD_STAGES": 3, "CHILL_TUNE_DQ_STAGES": 3}),
+    ("w8_s128", {"CHILL_TUNE_FWD_WAVES": 8, "CHILL_TUNE_DQ_WAVES": 8, "CHILL_TUNE_FWD_STREAMED": 128,
+                 "CHILL_TUNE_DQ_STREAMED": 128, "CHILL_TUNE_FWD_STAGES": 2, "CHILL_TUNE_DQ_STAGES": 2}),
+    # 4 waves, one workgroup per CU (three LDS stages)
+    ("w4_s64", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4, "CHILL_TUNE_FWD_STREAMED": 64,
+                "CHILL_TUNE_DQ_STREAMED": 64, "CHILL_TUNE_FWD_STAGES": 3, "CHILL_TUNE_DQ_STAGES": 3}),
+    # 4 waves, two workgroups per CU (two or three LDS stages of half the size)
+    ("w4_s64_n2", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4, "CHILL_TUNE_FWD_STREAMED": 64,
+                   "CHILL_TUNE_DQ_STREAMED": 64, "CHILL_TUNE_FWD_STAGES": 2, "CHILL_TUNE_DQ_STAGES": 2}),
+    ("w4_s32_n3", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4, "CHILL_TUNE_FWD_STREAMED": 32,
+                   "CHILL_TUNE_DQ_STREAMED": 32, "CHILL_TUNE_FWD_STAGES": 3, "CHILL_TUNE_DQ_STAGES": 3}),
     # dK/dV with 64 key rows per wave, K in registers and the accumulators in hand-managed accumulation
     # registers (head dims 64 and 128): as fast as the shipped paired kernel, not faster
     ("dkdv_r64", {"CHILL_TUNE_DKDV_R64": 1, "__flags__": "-mllvm -amdgpu-spill-vgpr-to-agpr=0"}),

@@ -105,8 +105,17 @@ __device__ __forceinline__ void softmax_grad_block(f32x16& s, f32x16& dp, float 
 // ------------------------------------------------------------------------------------------ dQ
 // Same skeleton as the forward kernel: asynchronous K/V ring, 32-key steps, the two score GEMMs of
 // step t+1 (S^T and dP^T) issued before the vector work of step t.
+// Workgroups of four waves whose LDS ring leaves room for a second workgroup on the CU are compiled
+// for 256 registers per wave, so that two of them share a CU: one computes while the other loads its
+// first tiles or stores its result.
+template <typename E, int D, int NW, int TK, int NS>
+constexpr int dq_waves_per_simd() {
+    return (NW == 4 && Elem<E>::k16 && 2 * NS * 2 * LdsTile<E, D>::bytes(TK) <= 160 * 1024) ? 2 : 1;
+}
+
 template <typename E, int D, int MASK, int NW, int TK, int NS>
-__global__ __launch_bounds__(NW * 64) void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(dq_waves_per_simd<E, D, NW, TK, NS>())))
+void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
                                                      int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     constexpr int TQ = NW * 32;
@@ -259,7 +268,7 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = dq_tile_config(MASK_ID, D, Elem<E>::kDType);
         static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
-        constexpr int NS = dq_stages_for(cfg.streamed, D, Elem<E>::kDType);
+        constexpr int NS = dq_stages(MASK_ID, D, Elem<E>::kDType);
         const int n_q_tiles = cdiv(p.T, cfg.rows);
         const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;

@@ -325,11 +325,20 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
 #include "chill_fwd_regs.h"
 namespace chill {
 
+// Workgroups of four waves whose LDS ring leaves room for a second workgroup on the CU are compiled
+// for 256 registers per wave, so that two of them share a CU: one computes while the other loads its
+// first tiles or stores its result.
+template <typename E, int D, int NW, int TK, int NS>
+constexpr int fwd_waves_per_simd() {
+    return (NW == 4 && Elem<E>::k16 && 2 * NS * FwdLds<E, D, TK>::STAGE_BYTES <= 160 * 1024) ? 2 : 1;
+}
+
 // One workgroup per (batch, head, PAIR of q-tiles): tile j from the end, then tile j from the
 // start.  For causal-like masks the work of a q-tile grows with its index, so the two halves of a
 // pair add up to the same amount for every workgroup and the grid finishes without a tail.
 template <typename E, int D, int MASK, int NW, int TK, int NS>
-__global__ __launch_bounds__(NW * 64) void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(fwd_waves_per_simd<E, D, NW, TK, NS>())))
+void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
                                                       int wave_has_full_blocks, int paired) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
@@ -364,7 +373,7 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
     CHILL_DISPATCH_MASK(mask_id, {
         constexpr TileConfig cfg = fwd_tile_config(MASK_ID, D, Elem<E>::kDType);
         static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
-        constexpr int NS = fwd_stages_for(cfg.streamed, D, Elem<E>::kDType);
+        constexpr int NS = fwd_stages(MASK_ID, D, Elem<E>::kDType);
         static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES,
                       "table and kernel disagree on LDS");
         const int n_q_tiles = cdiv(p.T, cfg.rows);

@@ -18,6 +18,12 @@
 #ifndef CHILL_TUNE_FWD_STREAMED
 #define CHILL_TUNE_FWD_STREAMED 0
 #endif
+#ifndef CHILL_TUNE_FWD_STAGES
+#define CHILL_TUNE_FWD_STAGES 0
+#endif
+#ifndef CHILL_TUNE_DQ_STAGES
+#define CHILL_TUNE_DQ_STAGES 0
+#endif
 #ifndef CHILL_TUNE_DQ_WAVES
 #define CHILL_TUNE_DQ_WAVES 0
 #endif
@@ -50,48 +56,82 @@ constexpr int fwd_stage_bytes(int streamed, int D, int dtype) {
     return streamed * (rb + 16) + streamed * (rb + vpad);
 }
 
-// LDS stages of the forward K/V ring: three (one tile resident ahead, one in flight) when they fit
-// in 144 KiB, else two.
-constexpr int fwd_stages_for(int streamed, int D, int dtype) {
-    return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
+// Masks whose rows see a narrow band of keys: a q-tile is a short loop, and the time a workgroup
+// spends before and after it (loading Q and the first K/V tile, storing O) is a large part of its
+// life.  They get workgroups of four waves with a two-stage ring, two of which share a CU, so that one
+// computes while the other loads or stores (measured: sliding window forward -22 %, dQ -16 %;
+// chunkwise forward -5 %, dQ -14 %; on the causal workload the same shape re-reads K and V twice as
+// often and is 1-2 % slower).
+constexpr bool mask_is_banded(int mask_id) {
+    return mask_id == CHILL_MASK_SLIDING_WINDOW || mask_id == CHILL_MASK_CHUNKWISE;
 }
 
-// Forward.  16-bit inputs, head dim <= 128: 8 waves (256 query rows).  Streamed tiles of 128 keys for
-// head dims 64 and 128 (half the barriers per key; measured -12 % at D = 64, -8 % on the chunkwise
-// configuration, equal on the causal one), except for the sliding window, whose narrow band pays
-// for every partially used tile: 64 keys.
+// Forward.  16-bit inputs, head dim <= 128: 8 waves (256 query rows), streamed tiles of 128 keys for
+// head dims 64 and 128 (half the barriers per key; measured -12 % at D = 64, equal on the causal
+// workload), 64 keys below; banded masks: 4 waves, 64 keys, 2 stages.
+constexpr int fwd_waves(int mask_id, int D, int dtype) {
+    if (dtype == CHILL_F32 || D > 128) return 4;
+    if (CHILL_TUNE_FWD_WAVES) return CHILL_TUNE_FWD_WAVES;
+    return mask_is_banded(mask_id) ? 4 : 8;
+}
+constexpr int fwd_streamed(int mask_id, int D, int dtype) {
+    if (dtype == CHILL_F32) return 32;
+    if (D > 128) return CHILL_TUNE_D256_STREAMED;
+    if (CHILL_TUNE_FWD_STREAMED) return CHILL_TUNE_FWD_STREAMED;
+    return (D >= 64 && !mask_is_banded(mask_id)) ? 128 : 64;
+}
+// LDS stages of the forward K/V ring: two for the 4-wave shape of 16-bit inputs (so that two
+// workgroups fit a CU); otherwise three (one tile resident ahead, one in flight) when they fit in
+// 144 KiB, else two.
+constexpr int fwd_stages(int mask_id, int D, int dtype) {
+    const int streamed = fwd_streamed(mask_id, D, dtype);
+    if (dtype != CHILL_F32 && D <= 128) {
+        if (CHILL_TUNE_FWD_STAGES) return CHILL_TUNE_FWD_STAGES;
+        if (fwd_waves(mask_id, D, dtype) == 4) return 2;
+    }
+    return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
+}
 // 16-bit inputs at head dim 256: fwd_regs_kernel (O^T in hand-managed accumulation registers).
 constexpr bool fwd_uses_regs(int D, int dtype) { return CHILL_TUNE_FWD_REGS && dtype != CHILL_F32 && D == 256; }
 
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
-    const bool fast16 = dtype != CHILL_F32 && D <= 128;
-    const int tuned_streamed = (D >= 64 && mask_id != CHILL_MASK_SLIDING_WINDOW) ? 128 : 64;
-    const int waves = fast16 ? (CHILL_TUNE_FWD_WAVES ? CHILL_TUNE_FWD_WAVES : 8) : 4;
-    const int wide16 = (dtype != CHILL_F32 && D == 256) ? CHILL_TUNE_D256_STREAMED : 32;
-    const int streamed = fast16 ? (CHILL_TUNE_FWD_STREAMED ? CHILL_TUNE_FWD_STREAMED : tuned_streamed) : wide16;
+    const int waves = fwd_waves(mask_id, D, dtype);
+    const int streamed = fwd_streamed(mask_id, D, dtype);
     return TileConfig{waves * 32, streamed, waves,
-                      fwd_stages_for(streamed, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
+                      fwd_stages(mask_id, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
 }
 
-// dQ LDS stage: swizzled (unpadded) K and V tiles; three stages when they fit in 144 KiB.
-constexpr int dq_stages_for(int streamed, int D, int dtype) {
-    return 3 * 2 * streamed * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
-}
-
-// dQ.  16-bit inputs, head dim <= 128: 8 waves x 64 streamed keys; for the sliding window at head
-// dim <= 64, 4 waves x 32 keys (measured -17 %: a 128-row workgroup spans fewer unused tiles).
-// 16-bit inputs at head dim 256: dq_regs_kernel (hand-managed accumulation registers), 4 waves,
+// dQ.  16-bit inputs, head dim <= 128: 8 waves x 64 streamed keys in three stages; banded masks and
+// head dims <= 64: 4 waves x 64 keys in two stages, two workgroups per CU (prefix-LM at D = 64: dQ
+// -9 %).  16-bit inputs at head dim 256: dq_regs_kernel (hand-managed accumulation registers), 4 waves,
 // dq_regs_keys streamed keys per tile (0: the shape is served by dq_kernel).
 constexpr int dq_regs_keys(int D, int dtype) { return (dtype != CHILL_F32 && D == 256) ? CHILL_TUNE_DQ_REGS_KEYS : 0; }
+constexpr int dq_waves(int mask_id, int D, int dtype) {
+    if (dtype == CHILL_F32 || D > 128) return 4;
+    if (CHILL_TUNE_DQ_WAVES) return CHILL_TUNE_DQ_WAVES;
+    return (mask_is_banded(mask_id) || D <= 64) ? 4 : 8;
+}
+constexpr int dq_streamed(int mask_id, int D, int dtype) {
+    (void)mask_id;
+    if (dtype == CHILL_F32) return 32;
+    if (D > 128) return dq_regs_keys(D, dtype) > 0 ? dq_regs_keys(D, dtype) : 32;
+    return CHILL_TUNE_DQ_STREAMED ? CHILL_TUNE_DQ_STREAMED : 64;
+}
+// dQ LDS stage: swizzled (unpadded) K and V tiles.  Two stages for the 4-wave shape of 16-bit inputs;
+// otherwise three when they fit in 144 KiB.
+constexpr int dq_stages(int mask_id, int D, int dtype) {
+    if (dtype != CHILL_F32 && D <= 128) {
+        if (CHILL_TUNE_DQ_STAGES) return CHILL_TUNE_DQ_STAGES;
+        if (dq_waves(mask_id, D, dtype) == 4) return 2;
+    }
+    return 3 * 2 * dq_streamed(mask_id, D, dtype) * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
+}
 
 constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
-    const bool fast16 = dtype != CHILL_F32 && D <= 128;
-    const int wide = dq_regs_keys(D, dtype) > 0 ? dq_regs_keys(D, dtype) : 32;
-    const bool narrow = mask_id == CHILL_MASK_SLIDING_WINDOW && D <= 64;
-    const int waves = fast16 ? (CHILL_TUNE_DQ_WAVES ? CHILL_TUNE_DQ_WAVES : (narrow ? 4 : 8)) : 4;
-    const int streamed = fast16 ? (CHILL_TUNE_DQ_STREAMED ? CHILL_TUNE_DQ_STREAMED : (narrow ? 32 : 64)) : wide;
+    const int waves = dq_waves(mask_id, D, dtype);
+    const int streamed = dq_streamed(mask_id, D, dtype);
     return TileConfig{waves * 32, streamed, waves,
-                      dq_stages_for(streamed, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
+                      dq_stages(mask_id, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
 }
 
 // dK/dV, rows of at most 256 bytes ("paired" kernel): a workgroup of 8 waves owns 128 key rows;

@@ -117,7 +117,13 @@ def test_tile_table():
     assert tile_config(causal, 64, torch.float16, _lib.PASS_FWD)["streamed"] == 128
     assert tile_config(causal, 32, torch.float16, _lib.PASS_FWD)["streamed"] == 64
     assert tile_config(window, 64, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 64
-    assert (tile_config(window, 64, torch.bfloat16, _lib.PASS_DQ)["waves"], tile_config(causal, 64, torch.bfloat16, _lib.PASS_DQ)["waves"]) == (4, 8)
+    # banded masks (and dQ at head dims <= 64): 4 waves with a two-stage ring, two workgroups per CU
+    for p, mask, D, waves in ((_lib.PASS_FWD, window, 64, 4), (_lib.PASS_FWD, window, 128, 4), (_lib.PASS_FWD, causal, 64, 8),
+                              (_lib.PASS_DQ, window, 128, 4), (_lib.PASS_DQ, causal, 64, 4), (_lib.PASS_DQ, causal, 128, 8)):
+        c = tile_config(mask, D, torch.bfloat16, p)
+        assert c["waves"] == waves, (p, D, c)
+        if waves == 4:
+            assert c["streamed"] == 64 and 2 * c["lds_bytes"] <= 160 * 1024
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
     assert tq == 32 * waves and tk % 32 == 0
     (dq_q, dq_k, _), (dk_q, dk_k, _) = _get_default_config_bwd(128, torch.bfloat16)
@@ -145,8 +151,8 @@ def test_tile_sweep_candidates():
 
     names = [n for n, _ in tune.CANDIDATES]
     assert len(set(names)) == len(names) and tune.CANDIDATES[0][1] == {}
-    allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_DQ_WAVES", "CHILL_TUNE_DQ_STREAMED",
-               "CHILL_TUNE_DKDV_R64", "__flags__"}
+    allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_FWD_STAGES", "CHILL_TUNE_DQ_WAVES",
+               "CHILL_TUNE_DQ_STREAMED", "CHILL_TUNE_DQ_STAGES", "CHILL_TUNE_DKDV_R64", "__flags__"}
     header = open(os.path.join(ROOT, "chill-attention_amd", "csrc", "chill_tiles.h")).read()
     for _, macros in tune.CANDIDATES:
         assert set(macros) <= allowed and all(m in header for m in macros if m != "__flags__")
