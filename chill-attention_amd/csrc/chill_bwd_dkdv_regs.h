@@ -201,11 +201,16 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
 #pragma unroll
             for (int c = 0; c < CB; c++) {
                 const int k_pos = kw + 32 * c + n;
+                if constexpr (Mask<MASK>::kRowIsRange) {
+                    const Range vis = visible_range<MASK, false>(k_pos, seq_len, p.margs);
+                    fill_outside_range(s[c], vis.lo, vis.hi, q0 + 4 * h, masked_score);
+                } else {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
-                    const bool ok = (q < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(q, k_pos, seq_len, p.margs);
-                    s[c][r] = ok ? s[c][r] : masked_score;
+                    for (int r = 0; r < 16; r++) {
+                        const int q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
+                        const bool ok = (q < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(q, k_pos, seq_len, p.margs);
+                        s[c][r] = ok ? s[c][r] : masked_score;
+                    }
                 }
             }
             // a row that attends to nothing has LSE2 = -inf and only masked entries

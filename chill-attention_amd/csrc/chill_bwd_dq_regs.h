@@ -96,6 +96,7 @@ __global__ __launch_bounds__(256) void dq_regs_kernel(BwdParams p, int n_q_tiles
     }
     // a row that attends to nothing has LSE2 = -inf and only masked entries (score -inf): P = exp2(-inf - 0)
     if (lse_q == -INFINITY) lse_q = 0.f;
+    const Range vis = visible_range<MASK, true>(q_pos, seq_len, p.margs);  // the keys this lane's row sees
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
@@ -148,11 +149,15 @@ __global__ __launch_bounds__(256) void dq_regs_kernel(BwdParams p, int n_q_tiles
             }
             mfma_fence(cs, cdp);
             if (!full) {
+                if constexpr (Mask<MASK>::kRowIsRange) {
+                    fill_outside_range(cs, vis.lo, vis.hi, k0 + 32 * kb + 4 * h, masked_score);
+                } else {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
-                    const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
-                    cs[r] = ok ? cs[r] : masked_score;
+                    for (int r = 0; r < 16; r++) {
+                        const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+                        const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
+                        cs[r] = ok ? cs[r] : masked_score;
+                    }
                 }
             }
 #pragma unroll

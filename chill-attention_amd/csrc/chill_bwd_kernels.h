@@ -187,6 +187,7 @@ void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
     }
     // a row that attends to nothing has LSE2 = -inf and only masked entries (score -inf): P = exp2(-inf - 0)
     if (lse_q == -INFINITY) lse_q = 0.f;
+    const Range vis = visible_range<MASK, true>(q_pos, seq_len, p.margs);  // the keys this lane's row sees
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
@@ -239,11 +240,15 @@ void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
             f32x16 cs, cdp;
             gemms(cs, cdp, stage, kb);
             if (!full) {
+                if constexpr (Mask<MASK>::kRowIsRange) {
+                    fill_outside_range(cs, vis.lo, vis.hi, k0 + 32 * kb + 4 * h, masked_score);
+                } else {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
-                    const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
-                    cs[r] = ok ? cs[r] : masked_score;
+                    for (int r = 0; r < 16; r++) {
+                        const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+                        const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
+                        cs[r] = ok ? cs[r] : masked_score;
+                    }
                 }
             }
 #pragma unroll
@@ -426,6 +431,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
 
     const int kw = kb0 + 32 * kblk;
     const int k_pos = kw + n;
+    const Range vis = visible_range<MASK, false>(k_pos, seq_len, p.margs);  // the queries that see this lane's key
     OperandOffsets<E, D> ofs;
     ofs.init(lane);
 
@@ -490,12 +496,19 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
             s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
         }
         if (!full) {
+            if constexpr (Mask<MASK>::kRowIsRange) {
+                fill_outside_range(s, vis.lo, vis.hi, q0 + 4 * h, masked_score);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
+                    const bool ok = (q < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(q, k_pos, seq_len, p.margs);
+                    s[r] = ok ? s[r] : masked_score;
+                }
+            }
+            // a row that attends to nothing has LSE2 = -inf and only masked entries
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int q = q0 + 8 * (r / 4) + 4 * h + (r % 4);
-                const bool ok = (q < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(q, k_pos, seq_len, p.margs);
-                s[r] = ok ? s[r] : masked_score;
-                // a row that attends to nothing has LSE2 = -inf and only masked entries
                 const float l = lse4[r / 4][r % 4];
                 lse4[r / 4][r % 4] = (l == -INFINITY) ? 0.f : l;
             }

@@ -238,6 +238,27 @@ __device__ __forceinline__ void mfma_fence(f32x16& x0, f32x16& x1) {
 }
 __device__ __forceinline__ void mfma_fence(f32x16& x0) { asm volatile("s_nop 11" : "+v"(x0)); }
 
+// Masking a 32 x 32 accumulator block by a range.  A lane holds, for its own row (or column) of the
+// block, the 16 entries at positions pos0 + 8 * (r / 4) + (r % 4) of the other axis, where pos0 = first
+// position of the block + 4 * (lane / 32).  Entries outside [lo, hi] become `fill`.  Most partial
+// blocks are cut on one side only (wave-uniform test), which leaves one comparison per entry.
+__device__ __forceinline__ void fill_outside_range(f32x16& s, int lo, int hi, int pos0, float fill) {
+    const int a = lo - pos0, b = hi - pos0;  // entry r is visible iff a <= c(r) <= b, c(r) = 8 * (r / 4) + (r % 4)
+    if (__builtin_amdgcn_ballot_w64(a > 0) == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = (8 * (r / 4) + (r % 4) <= b) ? s[r] : fill;
+    } else if (__builtin_amdgcn_ballot_w64(b < 27) == 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = (8 * (r / 4) + (r % 4) >= a) ? s[r] : fill;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int c = 8 * (r / 4) + (r % 4);
+            s[r] = (c >= a && c <= b) ? s[r] : fill;
+        }
+    }
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ------------------------------------------------------------------------------------------

@@ -111,6 +111,7 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
     float m_use = 0.f;        // m_run, or 0 while the row has seen no unmasked key
     float l_run = 0.f;        // this lane's share of the row sum
     const int q_pos = qw + n;
+    const Range vis = visible_range<MASK, true>(q_pos, seq_len, p.margs);  // the keys this lane's row sees
     // A negative scale reverses the order of the scores: the sign goes into Q, the softmax works
     // with |scale| (max(scale * s) = |scale| * max(sign * s)).
     const float scale = fabsf(p.scale_log2);
@@ -131,11 +132,15 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
     auto prepare = [&](f32x16& sc, bool full, int key0) -> float {
         mfma_fence(sc);
         if (!full) {
+            if constexpr (M::kRowIsRange) {
+                fill_outside_range(sc, vis.lo, vis.hi, key0 + 4 * h, -INFINITY);
+            } else {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
-                bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
-                sc[r] = ok ? sc[r] : -INFINITY;
+                for (int r = 0; r < 16; r++) {
+                    int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+                    bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
+                    sc[r] = ok ? sc[r] : -INFINITY;
+                }
             }
         }
         float mx = sc[0];

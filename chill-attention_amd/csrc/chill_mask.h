@@ -49,6 +49,10 @@ struct Mask;
 // What a mask functor inherits unless it says otherwise — the defaults of the reference's ChillMask
 // base class (mask.py:110-250): no predicate-free ranges, no full blocks, rows may be empty, and
 // limits that never decrease from one row to the next (the reference's *_lims_continious = True).
+// kRowIsRange = true states that the visible positions of a row ARE its range: pred(q, k) holds for
+// exactly the k in k_range_for_q(q) and exactly the q in q_range_for_k(k) (true of the five
+// built-in masks; the kernels then mask a partial block with two comparisons per entry instead of
+// evaluating the predicate).
 // A functor whose limits are NOT monotone sets kMonotoneLimits = false; tile ranges then come
 // from the minimum / maximum over the rows of a tile (utils.py:259-268).
 struct MaskDefaults {
@@ -57,6 +61,7 @@ struct MaskDefaults {
     static constexpr bool kHasKFullRange = false;
     static constexpr bool kHasQFullRange = false;
     static constexpr bool kMonotoneLimits = true;
+    static constexpr bool kRowIsRange = false;
     CHILL_HD static Range k_full_range_for_q(int, int, int, MaskArgs) { return {0, 0}; }
     CHILL_HD static Range q_full_range_for_k(int, int, int, MaskArgs) { return {0, 0}; }
     CHILL_HD static bool has_full_blocks(int, int, int, MaskArgs) { return false; }
@@ -70,6 +75,7 @@ struct Mask<CHILL_MASK_FULL> : MaskDefaults {
     static constexpr bool kSafe = true;        // every row sees at least one key (mask.py:864)
     static constexpr bool kHasKFullRange = true;
     static constexpr bool kHasQFullRange = true;
+    static constexpr bool kRowIsRange = true;
     CHILL_HD static bool pred(int, int, int, MaskArgs) { return true; }
     CHILL_HD static Range k_range_for_q(int, int seq_len, MaskArgs) { return {0, seq_len - 1}; }
     CHILL_HD static Range q_range_for_k(int, int seq_len, MaskArgs) { return {0, seq_len - 1}; }
@@ -86,6 +92,7 @@ struct Mask<CHILL_MASK_CAUSAL> : MaskDefaults {
     static constexpr bool kSafe = true;
     static constexpr bool kHasKFullRange = true;
     static constexpr bool kHasQFullRange = true;
+    static constexpr bool kRowIsRange = true;
     CHILL_HD static bool pred(int q, int k, int, MaskArgs) { return q >= k; }
     CHILL_HD static Range k_range_for_q(int q, int, MaskArgs) { return {0, q}; }
     CHILL_HD static Range q_range_for_k(int k, int seq_len, MaskArgs) { return {k, seq_len - 1}; }
@@ -109,6 +116,7 @@ struct Mask<CHILL_MASK_SLIDING_WINDOW> : MaskDefaults {
     static constexpr bool kSafe = false;
     static constexpr bool kHasKFullRange = true;
     static constexpr bool kHasQFullRange = true;
+    static constexpr bool kRowIsRange = true;
     CHILL_HD static bool pred(int q, int k, int, MaskArgs a) {
         return (k <= q + a.a1) & (k >= q - a.a0);
     }
@@ -152,6 +160,7 @@ struct Mask<CHILL_MASK_CHUNKWISE> : MaskDefaults {
     static constexpr bool kSafe = false;
     static constexpr bool kHasKFullRange = true;
     static constexpr bool kHasQFullRange = true;
+    static constexpr bool kRowIsRange = true;
     CHILL_HD static bool pred(int q, int k, int, MaskArgs a) {
         int d = q / a.a0 - k / a.a0;
         return (d >= 0) & (d <= a.a1);
@@ -199,6 +208,7 @@ struct Mask<CHILL_MASK_PREFIX_LM> : MaskDefaults {
     static constexpr bool kSafe = true;
     static constexpr bool kHasKFullRange = true;
     static constexpr bool kHasQFullRange = true;
+    static constexpr bool kRowIsRange = true;
     CHILL_HD static bool pred(int q, int k, int, MaskArgs a) { return (k < a.a0) | (q >= k); }
     CHILL_HD static Range k_range_for_q(int q, int seq_len, MaskArgs a) {
         return {0, imin(imax(q, a.a0 - 1), seq_len - 1)};
@@ -223,6 +233,15 @@ struct Mask<CHILL_MASK_PREFIX_LM> : MaskDefaults {
         return causal_full | in_prefix;
     }
 };
+
+// Visible positions of one row as an inclusive range clipped to the sequence (QROWS: the keys of
+// query `row`, else the queries of key `row`); empty (lo > hi) for a row past the end.
+template <int ID, bool QROWS>
+CHILL_HD Range visible_range(int row, int seq_len, MaskArgs a) {
+    if (row >= seq_len) return {1, 0};
+    const Range r = QROWS ? Mask<ID>::k_range_for_q(row, seq_len, a) : Mask<ID>::q_range_for_k(row, seq_len, a);
+    return {imax(r.lo, 0), imin(r.hi, seq_len - 1)};
+}
 
 // ---------------------------------------------------------------- tile decisions
 // Tiles of the streamed axis one row tile has to visit, and the sub-range of them that needs no

@@ -57,6 +57,25 @@ def test_make_mask_equals_oracle(m):
 
 
 @pytest.mark.parametrize("m", MASK_INSTANCES, ids=mask_id)
+def test_rows_and_columns_are_their_ranges(m):
+    """The kernels mask a partial block of a built-in mask by comparing positions with the row's
+    (column's) range instead of evaluating the predicate (kRowIsRange in csrc/chill_mask.h).  That is
+    only right if every row and column of the dense mask is exactly its range, without holes: checked
+    against the oracle's dense mask with the compiled limits."""
+    mask = make_mask(m)
+    desc = mask.descriptor()
+    for n in (1, 10, 33, 500, 1025):
+        dense = orc.dense_mask(m[0], m[1], n)
+        pos = np.arange(n)
+        for which, rows in ((0, dense), (1, dense.T)):
+            lim = np.zeros((n, 2), dtype=np.int32)
+            assert _lib.lib.chill_mask_limits(ctypes.byref(desc), which, n, n, lim.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))) == 0
+            lo = np.maximum(lim[:, 0], 0)[:, None]
+            hi = np.minimum(lim[:, 1], n - 1)[:, None]
+            assert ((pos[None, :] >= lo) & (pos[None, :] <= hi) == rows).all(), (m, n, which)
+
+
+@pytest.mark.parametrize("m", MASK_INSTANCES, ids=mask_id)
 def test_python_rules_equal_oracle(m):
     mask = make_mask(m)
     name, args = m
