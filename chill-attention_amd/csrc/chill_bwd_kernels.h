@@ -320,7 +320,8 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
     constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * VEC_BYTES;  // Q, dO, LSE2, delta
     constexpr int RING_OFF = 2 * KV_BYTES;                        // K, V tiles first
     static_assert(NS == 2, "two ring stages");
-    static_assert(DB * 16 * 256 * NKB <= RING_OFF + NS * STAGE_BYTES, "pair reduction reuses the LDS");
+    // the pair exchange at the end reuses the LDS: 2 * NKB accumulators of DB * 16 * 64 floats (the tile
+    // table allocates the larger of the two needs)
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
@@ -530,28 +531,66 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);  // dK^T += Q^T dS
     }
 
-    // sum the two waves of a pair through LDS (one accumulator at a time), then store
+    // Sum the two waves of a pair through LDS and store: the waves of the second half hand their dK^T
+    // partials to the first half and receive its dV^T partials, so that every wave finishes one 32 x D
+    // block.  The block then goes through LDS once more, row-major at a padded pitch, so that a store
+    // instruction writes whole rows (16 lanes x 16 bytes per 256-byte row) instead of 8 bytes of 32 rows.
     wait_async_tiles();
-    float* red = reinterpret_cast<float*>(smem) + kblk * (DB * 16 * 64) + lane;
-    auto reduce_and_store = [&](f32x16 (&acc)[DB], ET* base, int64_t row_stride, float mult) {
-        __syncthreads();  // everyone is done with the tiles (or with the previous round)
-        if (half == 1) {
+    constexpr int XCH_FLOATS = DB * 16 * 64;  // one wave's accumulator
+    float* xch_k = reinterpret_cast<float*>(smem) + kblk * XCH_FLOATS;
+    float* xch_v = reinterpret_cast<float*>(smem) + (NKB + kblk) * XCH_FLOATS;
+    f32x16(&give)[DB] = half == 1 ? dk : dv;
+    f32x16(&keep)[DB] = half == 1 ? dv : dk;
+    float* give_to = (half == 1 ? xch_k : xch_v) + lane;
+    float* take_from = (half == 1 ? xch_v : xch_k) + lane;
+    __syncthreads();  // everyone is done with the tiles
 #pragma unroll
-            for (int db = 0; db < DB; db++)
+    for (int db = 0; db < DB; db++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) red[(db * 16 + r) * 64] = acc[db][r];
+        for (int r = 0; r < 16; r++) give_to[(db * 16 + r) * 64] = give[db][r];
+    __syncthreads();
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) keep[db][r] += take_from[(db * 16 + r) * 64];
+
+    ET* out = half == 1 ? dvbase : dkbase;
+    const int64_t out_stride = half == 1 ? p.sdv.t : p.sdk.t;
+    const float mult = half == 1 ? 1.f : p.sm_scale;
+    const bool valid = k_pos < seq_len;
+    if constexpr (!Elem<E>::k16) {
+        if (k_pos < p.T) store_row_transposed<E, D>(out + (int64_t)k_pos * out_stride, keep, mult, valid, h);
+    } else {
+        // the region this wave just read is its own from here on: stage the finished block there
+        constexpr int RB = D * 2;       // bytes per row
+        constexpr int PITCH = RB + 8;   // 8-byte writes of 32 consecutive rows spread over all banks
+        constexpr int CH = RB / 16;     // 16-byte chunks per row
+        static_assert(32 * PITCH <= XCH_FLOATS * 4, "the staged block fits the wave's exchange region");
+        char* stage = reinterpret_cast<char*>(half == 1 ? xch_v : xch_k);
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d0 = 32 * db + 8 * g + 4 * h;
+                if (D >= 32 || d0 < D) {
+                    f32x4 vals;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) vals[e] = valid ? keep[db][4 * g + e] * mult : 0.f;
+                    *reinterpret_cast<i32x2*>(stage + n * PITCH + d0 * 2) = Elem<E>::pack4(vals);
+                }
+            }
+        constexpr int ROWS_PER_STEP = 64 / CH;  // 4 (D = 128) .. 32 (D = 16)
+#pragma unroll
+        for (int row0 = 0; row0 < 32; row0 += ROWS_PER_STEP) {
+            const int row = row0 + lane / CH, c = lane % CH;
+            // PITCH is a multiple of 8 only: two 8-byte reads
+            const i32x2 lo = *reinterpret_cast<const i32x2*>(stage + row * PITCH + c * 16);
+            const i32x2 hi = *reinterpret_cast<const i32x2*>(stage + row * PITCH + c * 16 + 8);
+            if (kw + row < p.T)
+                *reinterpret_cast<i32x4*>(reinterpret_cast<char*>(out + (int64_t)(kw + row) * out_stride) + c * 16) =
+                    i32x4{lo[0], lo[1], hi[0], hi[1]};
         }
-        __syncthreads();
-        if (half == 0) {
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) acc[db][r] += red[(db * 16 + r) * 64];
-            if (k_pos < p.T) store_row_transposed<E, D>(base + (int64_t)k_pos * row_stride, acc, mult, k_pos < seq_len, h);
-        }
-    };
-    reduce_and_store(dk, dkbase, p.sdk.t, p.sm_scale);
-    reduce_and_store(dv, dvbase, p.sdv.t, 1.f);
+    }
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV (wide rows)
@@ -768,6 +807,7 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
+        static_assert(!paired || cfg.lds_bytes >= dkdv_paired_exchange_bytes(D), "LDS for the pair exchange");
         void (*kern)(BwdParams, int, int, int);
         if constexpr (CB > 0)
             kern = dkdv_regs_kernel<E, D, MASK_ID, CB, dkdv_regs_stages(D)>;

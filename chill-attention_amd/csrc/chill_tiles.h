@@ -140,6 +140,9 @@ constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
 // Longer rows ("wide" kernel): 4 waves own 128 key rows with K, V resident in registers; the ring
 // holds 32-row Q and dO tiles.
 constexpr bool dkdv_is_paired(int D, int dtype) { return D * elem_bytes(dtype) <= 256; }
+// at the end the waves of a pair exchange one fp32 accumulator each through LDS: 8 waves x (D rounded
+// up to 32) x 32 floats
+constexpr int dkdv_paired_exchange_bytes(int D) { return 8 * ((D + 31) / 32) * 16 * 64 * 4; }
 constexpr int dkdv_wide_stage_bytes(int streamed, int D, int dtype) {
     return 2 * streamed * D * elem_bytes(dtype) + 2 * streamed * 4;
 }
@@ -168,8 +171,11 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
         const int rows = 4 * 32 * dkdv_regs_blocks(D, dtype);
         return TileConfig{rows, 32, 4, rows * row_bytes + dkdv_regs_stages(D) * (2 * 32 * row_bytes + 2 * 32 * 4)};
     }
-    if (dkdv_is_paired(D, dtype))
-        return TileConfig{128, 64, 8, 2 * 128 * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4)};
+    if (dkdv_is_paired(D, dtype)) {
+        const int ring = 2 * 128 * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4);
+        const int exchange = dkdv_paired_exchange_bytes(D);
+        return TileConfig{128, 64, 8, ring > exchange ? ring : exchange};
+    }
     return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
 }
 
