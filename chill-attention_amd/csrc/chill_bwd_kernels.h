@@ -279,8 +279,11 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        auto kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
-        if constexpr (dq_regs_keys(D, Elem<E>::kDType) > 0) kern = dq_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+        void (*kern)(BwdParams, int, int, int);
+        if constexpr (dq_regs_keys(D, Elem<E>::kDType) > 0)
+            kern = dq_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+        else
+            kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
         const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

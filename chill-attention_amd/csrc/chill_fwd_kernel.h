@@ -389,8 +389,11 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        auto kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
-        if constexpr (fwd_uses_regs(D, Elem<E>::kDType)) kern = fwd_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+        void (*kern)(FwdParams, int, int, int, int);
+        if constexpr (fwd_uses_regs(D, Elem<E>::kDType))
+            kern = fwd_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+        else
+            kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
         const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
         if (cfg.lds_bytes > 48 * 1024) {
             if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),

@@ -30,16 +30,6 @@
 #ifndef CHILL_TUNE_DQ_STREAMED
 #define CHILL_TUNE_DQ_STREAMED 0
 #endif
-
-#ifndef CHILL_TUNE_D256_STREAMED
-#define CHILL_TUNE_D256_STREAMED 64
-#endif
-#ifndef CHILL_TUNE_FWD_REGS
-#define CHILL_TUNE_FWD_REGS 1
-#endif
-#ifndef CHILL_TUNE_DQ_REGS_KEYS
-#define CHILL_TUNE_DQ_REGS_KEYS 32
-#endif
 #ifndef CHILL_TUNE_DKDV_R64
 #define CHILL_TUNE_DKDV_R64 0
 #endif
@@ -76,7 +66,7 @@ constexpr int fwd_waves(int mask_id, int D, int dtype) {
 }
 constexpr int fwd_streamed(int mask_id, int D, int dtype) {
     if (dtype == CHILL_F32) return 32;
-    if (D > 128) return CHILL_TUNE_D256_STREAMED;
+    if (D > 128) return 64;
     if (CHILL_TUNE_FWD_STREAMED) return CHILL_TUNE_FWD_STREAMED;
     return (D >= 64 && !mask_is_banded(mask_id)) ? 128 : 64;
 }
@@ -92,7 +82,7 @@ constexpr int fwd_stages(int mask_id, int D, int dtype) {
     return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
 // 16-bit inputs at head dim 256: fwd_regs_kernel (O^T in hand-managed accumulation registers).
-constexpr bool fwd_uses_regs(int D, int dtype) { return CHILL_TUNE_FWD_REGS && dtype != CHILL_F32 && D == 256; }
+constexpr bool fwd_uses_regs(int D, int dtype) { return dtype != CHILL_F32 && D == 256; }
 
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
     const int waves = fwd_waves(mask_id, D, dtype);
@@ -105,7 +95,7 @@ constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
 // head dims <= 64: 4 waves x 64 keys in two stages, two workgroups per CU (prefix-LM at D = 64: dQ
 // -9 %).  16-bit inputs at head dim 256: dq_regs_kernel (hand-managed accumulation registers), 4 waves,
 // dq_regs_keys streamed keys per tile (0: the shape is served by dq_kernel).
-constexpr int dq_regs_keys(int D, int dtype) { return (dtype != CHILL_F32 && D == 256) ? CHILL_TUNE_DQ_REGS_KEYS : 0; }
+constexpr int dq_regs_keys(int D, int dtype) { return (dtype != CHILL_F32 && D == 256) ? 32 : 0; }
 constexpr int dq_waves(int mask_id, int D, int dtype) {
     if (dtype == CHILL_F32 || D > 128) return 4;
     if (CHILL_TUNE_DQ_WAVES) return CHILL_TUNE_DQ_WAVES;
