@@ -50,6 +50,8 @@ WORKLOADS = {
     "C4": ("ChunkwiseChillMask", (128, 2), "f16", 2, 32, 16384, 128, 3, 0.5),
     "C5a": ("PrefixLMChillMask", (1024,), "bf16", 4, 32, 8192, 64, 4, 1.0),
     "C5b": ("PrefixLMChillMask", (1024,), "f32", 1, 8, 2048, 64, 4, 1.0),
+    # not a BASELINE configuration: the widest head dim, for inspecting its kernels
+    "D256": ("CausalChillMask", (), "bf16", 4, 8, 8192, 256, 5, 1.0),
 }
 
 
