@@ -276,6 +276,33 @@ def test_delta_kernel(D, dtype):
     np.testing.assert_allclose(delta.cpu().numpy(), want, atol=2e-5 * D, rtol=1e-5)
 
 
+@pytest.mark.parametrize("T,D,dtype", [(70001, 64, torch.float16), (100003, 128, torch.bfloat16)])
+def test_long_sequences(T, D, dtype):
+    """Sequences far beyond the BASELINE sizes, of a length no tile divides (row offsets past 2^24 elements):
+    O on row slices at the start, the middle and the end against dense fp32 attention over all keys, and the
+    scale symmetry sum(dQ . Q) == sum(dK . K) of the gradients."""
+    torch.manual_seed(0)
+    q, k, v = (torch.randn(1, 2, T, D, device=DEV, dtype=dtype, requires_grad=True) for _ in range(3))
+    do = torch.randn(1, 2, T, D, device=DEV, dtype=dtype)
+    ki = torch.arange(T, device=DEV)[None, :]
+    for mask, visible in (
+        (ca.CausalChillMask(), lambda qi: ki <= qi),
+        (ca.SlidingWindowChillMask(1000, 0), lambda qi: (ki <= qi) & (ki >= qi - 1000)),
+        (ca.PrefixLMChillMask(5000), lambda qi: (ki < 5000) | (ki <= qi)),
+    ):
+        o = ca.chill_attention(q, k, v, mask=mask)
+        dq, dk, dv = torch.autograd.grad(o, (q, k, v), do)
+        assert all(torch.isfinite(x).all().item() for x in (o, dq, dk, dv)), mask
+        for r0 in (0, T // 2 - 100, T - 300):
+            qi = torch.arange(r0, r0 + 300, device=DEV)[:, None]
+            scores = q[0, :, r0 : r0 + 300].float() @ k[0].float().transpose(-1, -2) * D**-0.5
+            ref = torch.softmax(scores.masked_fill(~visible(qi), float("-inf")), -1) @ v[0].float()
+            torch.testing.assert_close(o[0, :, r0 : r0 + 300].float(), ref, atol=1e-2, rtol=1e-2)
+        a = (dq.double() * q.double()).sum().item()
+        b = (dk.double() * k.double()).sum().item()
+        assert abs(a - b) <= 2e-2 * max(abs(a), abs(b), 1.0), (mask, a, b)
+
+
 def test_device_functors_equal_host():
     """The mask functors and tile decisions as executed ON THE GPU equal the host build bit for bit."""
     import ctypes
