@@ -307,7 +307,7 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
 // 32 x D accumulators, no resident MFMA operands) within 256 registers, so two waves share a SIMD
 // and one wave's vector work hides behind the other's MFMAs, with no redundant MFMA work.
 template <typename E, int D, int MASK, int NW, int NS>
-__global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4 ? 2 : 1))) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
                                                        int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     typedef LdsTile<E, D> L;
@@ -473,7 +473,7 @@ __global__ __launch_bounds__(NW * 64) void dkdv_kernel(BwdParams p, int n_k_tile
         if (!issue_late) {
             if (it + 1 < n_iters) issue_next(st_next);
         }
-        if (tile < ta || tile >= tb) continue;
+        if (!in_block) continue;
         const lds_char* q_tile = lds0 + RING_OFF + st_cur * STAGE_BYTES;
         const lds_char* do_tile = q_tile + TILE_BYTES;
         const lds_float* vec = reinterpret_cast<const lds_float*>(q_tile + 2 * TILE_BYTES) + 32 * half;
@@ -810,7 +810,7 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
         if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
         const int total = (int)total64;
         dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        static_assert(!paired || cfg.lds_bytes >= dkdv_paired_exchange_bytes(D), "LDS for the pair exchange");
+        static_assert(!paired || cfg.lds_bytes >= dkdv_paired_exchange_bytes(D) * cfg.waves / 8, "LDS for the pair exchange");
         void (*kern)(BwdParams, int, int, int);
         if constexpr (CB > 0)
             kern = dkdv_regs_kernel<E, D, MASK_ID, CB, dkdv_regs_stages(D)>;

@@ -30,6 +30,9 @@
 #ifndef CHILL_TUNE_DQ_STREAMED
 #define CHILL_TUNE_DQ_STREAMED 0
 #endif
+#ifndef CHILL_TUNE_DKDV_WAVES
+#define CHILL_TUNE_DKDV_WAVES 0
+#endif
 #ifndef CHILL_TUNE_DKDV_R64
 #define CHILL_TUNE_DKDV_R64 0
 #endif
@@ -130,6 +133,16 @@ constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
 // Longer rows ("wide" kernel): 4 waves own 128 key rows with K, V resident in registers; the ring
 // holds 32-row Q and dO tiles.
 constexpr bool dkdv_is_paired(int D, int dtype) { return D * elem_bytes(dtype) <= 256; }
+// 16-bit head dims <= 64: workgroups of 4 waves (64 key rows), small enough in LDS (50 KiB at D = 64)
+// and registers (167) for two or three of them per CU, which hide each other's start and end
+// (measured: sliding window dK/dV -32 %, prefix-LM at D = 64 -17 %).  At D = 128 the two-stage ring of
+// such a workgroup takes 99 KiB; with a one-stage ring it fits twice but runs 8 % slower than the
+// 8-wave workgroup.
+constexpr int dkdv_paired_waves(int mask_id, int D, int dtype) {
+    (void)mask_id;
+    if (CHILL_TUNE_DKDV_WAVES) return CHILL_TUNE_DKDV_WAVES;
+    return (dtype != CHILL_F32 && D <= 64) ? 4 : 8;
+}
 // at the end the waves of a pair exchange one fp32 accumulator each through LDS: 8 waves x (D rounded
 // up to 32) x 32 floats
 constexpr int dkdv_paired_exchange_bytes(int D) { return 8 * ((D + 31) / 32) * 16 * 64 * 4; }
@@ -155,16 +168,17 @@ constexpr int dkdv_regs_blocks(int D, int dtype) {
 constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
 
 constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
-    (void)mask_id;
     const int row_bytes = D * elem_bytes(dtype);
     if (dkdv_regs_blocks(D, dtype) > 0) {
         const int rows = 4 * 32 * dkdv_regs_blocks(D, dtype);
         return TileConfig{rows, 32, 4, rows * row_bytes + dkdv_regs_stages(D) * (2 * 32 * row_bytes + 2 * 32 * 4)};
     }
     if (dkdv_is_paired(D, dtype)) {
-        const int ring = 2 * 128 * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4);
-        const int exchange = dkdv_paired_exchange_bytes(D);
-        return TileConfig{128, 64, 8, ring > exchange ? ring : exchange};
+        const int waves = dkdv_paired_waves(mask_id, D, dtype);
+        const int rows = 16 * waves;
+        const int ring = 2 * rows * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4);
+        const int exchange = dkdv_paired_exchange_bytes(D) * waves / 8;
+        return TileConfig{rows, 64, waves, ring > exchange ? ring : exchange};
     }
     return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
 }

@@ -124,6 +124,11 @@ def test_tile_table():
         assert c["waves"] == waves, (p, D, c)
         if waves == 4:
             assert c["streamed"] == 64 and 2 * c["lds_bytes"] <= 160 * 1024
+    # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU
+    for D, rows, waves in ((64, 64, 4), (32, 64, 4), (128, 128, 8)):
+        c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV)
+        assert (c["rows"], c["waves"]) == (rows, waves), (D, c)
+    assert 2 * tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV)["lds_bytes"] <= 160 * 1024
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
     assert tq == 32 * waves and tk % 32 == 0
     (dq_q, dq_k, _), (dk_q, dk_k, _) = _get_default_config_bwd(128, torch.bfloat16)
@@ -152,7 +157,7 @@ def test_tile_sweep_candidates():
     names = [n for n, _ in tune.CANDIDATES]
     assert len(set(names)) == len(names) and tune.CANDIDATES[0][1] == {}
     allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_FWD_STAGES", "CHILL_TUNE_DQ_WAVES",
-               "CHILL_TUNE_DQ_STREAMED", "CHILL_TUNE_DQ_STAGES", "CHILL_TUNE_DKDV_R64", "__flags__"}
+               "CHILL_TUNE_DQ_STREAMED", "CHILL_TUNE_DQ_STAGES", "CHILL_TUNE_DKDV_WAVES", "CHILL_TUNE_DKDV_R64", "__flags__"}
     header = open(os.path.join(ROOT, "chill-attention_amd", "csrc", "chill_tiles.h")).read()
     for _, macros in tune.CANDIDATES:
         assert set(macros) <= allowed and all(m in header for m in macros if m != "__flags__")
