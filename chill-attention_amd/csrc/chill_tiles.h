@@ -59,19 +59,19 @@ constexpr bool mask_is_banded(int mask_id) {
     return mask_id == CHILL_MASK_SLIDING_WINDOW || mask_id == CHILL_MASK_CHUNKWISE;
 }
 
-// Forward.  16-bit inputs, head dim <= 128: 8 waves (256 query rows), streamed tiles of 128 keys for
-// head dims 64 and 128 (half the barriers per key; measured -12 % at D = 64, equal on the causal
-// workload), 64 keys below; banded masks: 4 waves, 64 keys, 2 stages.
+// Forward.  16-bit inputs at head dim 128: 8 waves (256 query rows), streamed tiles of 128 keys (half
+// the barriers per key); banded masks and head dims <= 64: 4 waves, 64 keys, 2 stages, two or three
+// workgroups per CU (prefix-LM at D = 64: forward -14 %; causal at D = 16 .. 64: -5 .. -8 %).
 constexpr int fwd_waves(int mask_id, int D, int dtype) {
     if (dtype == CHILL_F32 || D > 128) return 4;
     if (CHILL_TUNE_FWD_WAVES) return CHILL_TUNE_FWD_WAVES;
-    return mask_is_banded(mask_id) ? 4 : 8;
+    return (mask_is_banded(mask_id) || D <= 64) ? 4 : 8;
 }
 constexpr int fwd_streamed(int mask_id, int D, int dtype) {
     if (dtype == CHILL_F32) return 32;
     if (D > 128) return 64;
     if (CHILL_TUNE_FWD_STREAMED) return CHILL_TUNE_FWD_STREAMED;
-    return (D >= 64 && !mask_is_banded(mask_id)) ? 128 : 64;
+    return (D > 64 && !mask_is_banded(mask_id)) ? 128 : 64;
 }
 // LDS stages of the forward K/V ring: two for the 4-wave shape of 16-bit inputs (so that two
 // workgroups fit a CU); otherwise three (one tile resident ahead, one in flight) when they fit in

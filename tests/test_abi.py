@@ -114,11 +114,11 @@ def test_tile_table():
     # rows the tile sweep put into the table (mask- and head-dim-specific)
     causal, window = ca.CausalChillMask(), ca.SlidingWindowChillMask(128, 128)
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 128
-    assert tile_config(causal, 64, torch.float16, _lib.PASS_FWD)["streamed"] == 128
+    assert tile_config(causal, 64, torch.float16, _lib.PASS_FWD)["streamed"] == 64
     assert tile_config(causal, 32, torch.float16, _lib.PASS_FWD)["streamed"] == 64
     assert tile_config(window, 64, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 64
-    # banded masks (and dQ at head dims <= 64): 4 waves with a two-stage ring, two workgroups per CU
-    for p, mask, D, waves in ((_lib.PASS_FWD, window, 64, 4), (_lib.PASS_FWD, window, 128, 4), (_lib.PASS_FWD, causal, 64, 8),
+    # banded masks, and every mask at head dims <= 64: 4 waves with a two-stage ring, two or more workgroups per CU
+    for p, mask, D, waves in ((_lib.PASS_FWD, window, 64, 4), (_lib.PASS_FWD, window, 128, 4), (_lib.PASS_FWD, causal, 64, 4), (_lib.PASS_FWD, causal, 128, 8),
                               (_lib.PASS_DQ, window, 128, 4), (_lib.PASS_DQ, causal, 64, 4), (_lib.PASS_DQ, causal, 128, 8)):
         c = tile_config(mask, D, torch.bfloat16, p)
         assert c["waves"] == waves, (p, D, c)
