@@ -117,15 +117,17 @@ def run_case(provider, mode, mask, shape, T, dtype, use_graph, check):
     note = ""
     if check:
         # the reference's checks (benchmark.py:216-239): O within 3e-3, gradients within 1e-2 of the
-        # dense-mask SDPA result on the same inputs
-        ref, res_mask = ca._chill_reference_naive(mask, q, k, v, None)
+        # dense-mask SDPA result on the same inputs.  The oracle runs on fp32 copies of the inputs: in
+        # fp16 PyTorch's dense-mask kernel is itself up to 3.5e-3 away from the fp32 result on these
+        # inputs, which makes the 3e-3 check fail now and then whatever is being checked.
+        ref, res_mask = ca._chill_reference_naive(mask, q.float(), k.float(), v.float(), None)
         out = fn()
-        torch.testing.assert_close(out * res_mask.broadcast_to(out.shape), ref, atol=3e-3, rtol=0)
+        torch.testing.assert_close((out * res_mask.broadcast_to(out.shape)).float(), ref, atol=3e-3, rtol=0)
         if mode == "bwd" and provider != "flex":
             grads_ref = torch.autograd.grad(ref, (q, k, v), do.to(ref.dtype) * res_mask)
             grads = torch.autograd.grad(out, (q, k, v), do.to(out.dtype) * res_mask)
             for g, gr in zip(grads, grads_ref):
-                torch.testing.assert_close(g, gr, atol=1e-2, rtol=0)
+                torch.testing.assert_close(g.float(), gr.float(), atol=1e-2, rtol=0)
         del ref, out
         note = "checked"
     if mode == "fwd":
