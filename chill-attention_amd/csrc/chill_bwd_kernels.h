@@ -265,33 +265,48 @@ void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
         store_row_transposed<E, D>(dqbase + (int64_t)q_pos * p.sdq.t, dq, p.sm_scale, q_pos < seq_len, h);
 }
 
+// One (mask, tile shape): SHORT selects the table row for short sequences.
+template <typename E, int D, int MASK_ID, bool SHORT>
+int launch_dq_shape(const BwdParams& p, hipStream_t stream) {
+    constexpr int kRowFor = SHORT ? 1 : kLongSequence;
+    constexpr TileConfig cfg = dq_tile_config(MASK_ID, D, Elem<E>::kDType, kRowFor);
+    static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+    constexpr int NS = dq_stages(MASK_ID, D, Elem<E>::kDType, kRowFor);
+    const int n_q_tiles = cdiv(p.T, cfg.rows);
+    const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
+    if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
+    const int total = (int)total64;
+    dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
+    void (*kern)(BwdParams, int, int, int);
+    if constexpr (dq_regs_keys(D, Elem<E>::kDType) > 0)
+        kern = dq_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+    else
+        kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
+    const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
+    if (cfg.lds_bytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                cfg.lds_bytes) != hipSuccess)
+            return CHILL_ERR_HIP;
+    }
+    hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
+    return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+}
+
 template <typename E, int D>
 int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
     const int64_t max_stride = p.sk.t > p.sv.t ? p.sk.t : p.sv.t;
     if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
-        constexpr TileConfig cfg = dq_tile_config(MASK_ID, D, Elem<E>::kDType);
-        static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
-        constexpr int NS = dq_stages(MASK_ID, D, Elem<E>::kDType);
-        const int n_q_tiles = cdiv(p.T, cfg.rows);
-        const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
-        if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
-        const int total = (int)total64;
-        dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        void (*kern)(BwdParams, int, int, int);
-        if constexpr (dq_regs_keys(D, Elem<E>::kDType) > 0)
-            kern = dq_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
-        else
-            kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
-        const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
-        if (cfg.lds_bytes > 48 * 1024) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)
-                return CHILL_ERR_HIP;
+        // the table has a row of its own for short sequences where that row differs
+        constexpr bool has_short_row = dq_tile_config(MASK_ID, D, Elem<E>::kDType, 1).waves !=
+                                       dq_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
+        if constexpr (has_short_row) {
+            status = p.T <= kDqShortSequence ? launch_dq_shape<E, D, MASK_ID, true>(p, stream)
+                                             : launch_dq_shape<E, D, MASK_ID, false>(p, stream);
+        } else {
+            status = launch_dq_shape<E, D, MASK_ID, false>(p, stream);
         }
-        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
-        status = (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
     });
     return status;
 }

@@ -369,6 +369,37 @@ void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
 // shapes: 16-35 % faster below the threshold, 7-16 % slower at two to four times it)
 constexpr int kPairedMinWorkgroups = 256;
 
+// One (mask, tile shape): SHORT selects the table row for short sequences.
+template <typename E, int D, int MASK_ID, bool SHORT>
+int launch_fwd_shape(const FwdParams& p, hipStream_t stream) {
+    constexpr int kRowFor = SHORT ? 1 : kLongSequence;
+    constexpr TileConfig cfg = fwd_tile_config(MASK_ID, D, Elem<E>::kDType, kRowFor);
+    static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+    constexpr int NS = fwd_stages(MASK_ID, D, Elem<E>::kDType, kRowFor);
+    static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES, "table and kernel disagree on LDS");
+    const int n_q_tiles = cdiv(p.T, cfg.rows);
+    // pairing q-tiles balances long causal runs; with few workgroups it only halves the number of
+    // CUs that get work
+    const bool paired = (int64_t)p.B * p.H * ((n_q_tiles + 1) / 2) >= kPairedMinWorkgroups;
+    const int64_t total64 = (int64_t)p.B * p.H * (paired ? (n_q_tiles + 1) / 2 : n_q_tiles);
+    if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
+    const int total = (int)total64;
+    dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
+    void (*kern)(FwdParams, int, int, int, int);
+    if constexpr (fwd_uses_regs(D, Elem<E>::kDType))
+        kern = fwd_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+    else
+        kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
+    const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
+    if (cfg.lds_bytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                cfg.lds_bytes) != hipSuccess)
+            return CHILL_ERR_HIP;
+    }
+    hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0, paired ? 1 : 0);
+    return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+}
+
 template <typename E, int D>
 int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
     // the async loader keeps per-lane global offsets in 32 bits
@@ -376,32 +407,15 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
     if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
-        constexpr TileConfig cfg = fwd_tile_config(MASK_ID, D, Elem<E>::kDType);
-        static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
-        constexpr int NS = fwd_stages(MASK_ID, D, Elem<E>::kDType);
-        static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES,
-                      "table and kernel disagree on LDS");
-        const int n_q_tiles = cdiv(p.T, cfg.rows);
-        // pairing q-tiles balances long causal runs; with few workgroups it only halves the number of
-        // CUs that get work
-        const bool paired = (int64_t)p.B * p.H * ((n_q_tiles + 1) / 2) >= kPairedMinWorkgroups;
-        const int64_t total64 = (int64_t)p.B * p.H * (paired ? (n_q_tiles + 1) / 2 : n_q_tiles);
-        if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
-        const int total = (int)total64;
-        dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        void (*kern)(FwdParams, int, int, int, int);
-        if constexpr (fwd_uses_regs(D, Elem<E>::kDType))
-            kern = fwd_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
-        else
-            kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
-        const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
-        if (cfg.lds_bytes > 48 * 1024) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)
-                return CHILL_ERR_HIP;
+        // the table has a row of its own for short sequences where that row differs
+        constexpr bool has_short_row = fwd_tile_config(MASK_ID, D, Elem<E>::kDType, 1).waves !=
+                                       fwd_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
+        if constexpr (has_short_row) {
+            status = p.T <= kFwdShortSequence ? launch_fwd_shape<E, D, MASK_ID, true>(p, stream)
+                                              : launch_fwd_shape<E, D, MASK_ID, false>(p, stream);
+        } else {
+            status = launch_fwd_shape<E, D, MASK_ID, false>(p, stream);
         }
-        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0, paired ? 1 : 0);
-        status = (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
     });
     return status;
 }

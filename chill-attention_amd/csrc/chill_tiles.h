@@ -59,72 +59,81 @@ constexpr bool mask_is_banded(int mask_id) {
     return mask_id == CHILL_MASK_SLIDING_WINDOW || mask_id == CHILL_MASK_CHUNKWISE;
 }
 
+// Sequence lengths up to which the 4-wave shape also wins at head dim 128 for masks that are not banded
+// (measured on causal and full masks, B8 H4 .. H16: forward -16 % at T = 512 and 1024, +20 % at 2085;
+// dQ -24 % at 512, -14 % at 2048 and 4042, -5 % at 4096, +-1 % at 8192, where its extra K / V reads cost
+// the neighbouring kernels more than it gains).  T = kLongSequence selects the long-sequence row.
+constexpr int kLongSequence = 0x7fffffff;
+constexpr int kFwdShortSequence = 1024;
+constexpr int kDqShortSequence = 4096;
+
 // Forward.  16-bit inputs at head dim 128: 8 waves (256 query rows), streamed tiles of 128 keys (half
-// the barriers per key); banded masks and head dims <= 64: 4 waves, 64 keys, 2 stages, two or three
-// workgroups per CU (prefix-LM at D = 64: forward -14 %; causal at D = 16 .. 64: -5 .. -8 %).
-constexpr int fwd_waves(int mask_id, int D, int dtype) {
+// the barriers per key); banded masks, head dims <= 64 and short sequences: 4 waves, 64 keys, 2
+// stages, two or three workgroups per CU (prefix-LM at D = 64: forward -14 %; causal at D = 16 .. 64:
+// -5 .. -8 %).
+constexpr int fwd_waves(int mask_id, int D, int dtype, int T) {
     if (dtype == CHILL_F32 || D > 128) return 4;
     if (CHILL_TUNE_FWD_WAVES) return CHILL_TUNE_FWD_WAVES;
-    return (mask_is_banded(mask_id) || D <= 64) ? 4 : 8;
+    return (mask_is_banded(mask_id) || D <= 64 || T <= kFwdShortSequence) ? 4 : 8;
 }
-constexpr int fwd_streamed(int mask_id, int D, int dtype) {
+constexpr int fwd_streamed(int mask_id, int D, int dtype, int T) {
     if (dtype == CHILL_F32) return 32;
     if (D > 128) return 64;
     if (CHILL_TUNE_FWD_STREAMED) return CHILL_TUNE_FWD_STREAMED;
-    return (D > 64 && !mask_is_banded(mask_id)) ? 128 : 64;
+    return fwd_waves(mask_id, D, dtype, T) == 8 ? 128 : 64;
 }
 // LDS stages of the forward K/V ring: two for the 4-wave shape of 16-bit inputs (so that two
 // workgroups fit a CU); otherwise three (one tile resident ahead, one in flight) when they fit in
 // 144 KiB, else two.
-constexpr int fwd_stages(int mask_id, int D, int dtype) {
-    const int streamed = fwd_streamed(mask_id, D, dtype);
+constexpr int fwd_stages(int mask_id, int D, int dtype, int T) {
+    const int streamed = fwd_streamed(mask_id, D, dtype, T);
     if (dtype != CHILL_F32 && D <= 128) {
         if (CHILL_TUNE_FWD_STAGES) return CHILL_TUNE_FWD_STAGES;
-        if (fwd_waves(mask_id, D, dtype) == 4) return 2;
+        if (fwd_waves(mask_id, D, dtype, T) == 4) return 2;
     }
     return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
 // 16-bit inputs at head dim 256: fwd_regs_kernel (O^T in hand-managed accumulation registers).
 constexpr bool fwd_uses_regs(int D, int dtype) { return dtype != CHILL_F32 && D == 256; }
 
-constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype) {
-    const int waves = fwd_waves(mask_id, D, dtype);
-    const int streamed = fwd_streamed(mask_id, D, dtype);
+constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {
+    const int waves = fwd_waves(mask_id, D, dtype, T);
+    const int streamed = fwd_streamed(mask_id, D, dtype, T);
     return TileConfig{waves * 32, streamed, waves,
-                      fwd_stages(mask_id, D, dtype) * fwd_stage_bytes(streamed, D, dtype)};
+                      fwd_stages(mask_id, D, dtype, T) * fwd_stage_bytes(streamed, D, dtype)};
 }
 
-// dQ.  16-bit inputs, head dim <= 128: 8 waves x 64 streamed keys in three stages; banded masks and
-// head dims <= 64: 4 waves x 64 keys in two stages, two workgroups per CU (prefix-LM at D = 64: dQ
-// -9 %).  16-bit inputs at head dim 256: dq_regs_kernel (hand-managed accumulation registers), 4 waves,
-// dq_regs_keys streamed keys per tile (0: the shape is served by dq_kernel).
+// dQ.  16-bit inputs at head dim 128: 8 waves x 64 streamed keys in three stages; banded masks, head
+// dims <= 64 and sequences up to kDqShortSequence: 4 waves x 64 keys in two stages, two workgroups per
+// CU (prefix-LM at D = 64: dQ -9 %).  16-bit inputs at head dim 256: dq_regs_kernel (hand-managed
+// accumulation registers), 4 waves, dq_regs_keys streamed keys per tile (0: the shape is served by
+// dq_kernel).
 constexpr int dq_regs_keys(int D, int dtype) { return (dtype != CHILL_F32 && D == 256) ? 32 : 0; }
-constexpr int dq_waves(int mask_id, int D, int dtype) {
+constexpr int dq_waves(int mask_id, int D, int dtype, int T) {
     if (dtype == CHILL_F32 || D > 128) return 4;
     if (CHILL_TUNE_DQ_WAVES) return CHILL_TUNE_DQ_WAVES;
-    return (mask_is_banded(mask_id) || D <= 64) ? 4 : 8;
+    return (mask_is_banded(mask_id) || D <= 64 || T <= kDqShortSequence) ? 4 : 8;
 }
-constexpr int dq_streamed(int mask_id, int D, int dtype) {
-    (void)mask_id;
+constexpr int dq_streamed(int D, int dtype) {
     if (dtype == CHILL_F32) return 32;
     if (D > 128) return dq_regs_keys(D, dtype) > 0 ? dq_regs_keys(D, dtype) : 32;
     return CHILL_TUNE_DQ_STREAMED ? CHILL_TUNE_DQ_STREAMED : 64;
 }
 // dQ LDS stage: swizzled (unpadded) K and V tiles.  Two stages for the 4-wave shape of 16-bit inputs;
 // otherwise three when they fit in 144 KiB.
-constexpr int dq_stages(int mask_id, int D, int dtype) {
+constexpr int dq_stages(int mask_id, int D, int dtype, int T) {
     if (dtype != CHILL_F32 && D <= 128) {
         if (CHILL_TUNE_DQ_STAGES) return CHILL_TUNE_DQ_STAGES;
-        if (dq_waves(mask_id, D, dtype) == 4) return 2;
+        if (dq_waves(mask_id, D, dtype, T) == 4) return 2;
     }
-    return 3 * 2 * dq_streamed(mask_id, D, dtype) * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
+    return 3 * 2 * dq_streamed(D, dtype) * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
 }
 
-constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype) {
-    const int waves = dq_waves(mask_id, D, dtype);
-    const int streamed = dq_streamed(mask_id, D, dtype);
+constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {
+    const int waves = dq_waves(mask_id, D, dtype, T);
+    const int streamed = dq_streamed(D, dtype);
     return TileConfig{waves * 32, streamed, waves,
-                      dq_stages(mask_id, D, dtype) * 2 * streamed * D * elem_bytes(dtype)};
+                      dq_stages(mask_id, D, dtype, T) * 2 * streamed * D * elem_bytes(dtype)};
 }
 
 // dK/dV, rows of at most 256 bytes ("paired" kernel): a workgroup of 8 waves owns 128 key rows;
@@ -183,12 +192,14 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
     return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
 }
 
-inline int tile_config(int mask_id, int D, int dtype, int pass, TileConfig* out) {
+// T = sequence length the launch is for (the forward and dQ rows depend on it), kLongSequence for the
+// long-sequence row.
+inline int tile_config(int mask_id, int D, int dtype, int pass, int T, TileConfig* out) {
     if (dtype != CHILL_F32 && dtype != CHILL_F16 && dtype != CHILL_BF16) return CHILL_ERR_BAD_DTYPE;
     if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
     switch (pass) {
-        case CHILL_PASS_FWD: *out = fwd_tile_config(mask_id, D, dtype); return CHILL_OK;
-        case CHILL_PASS_DQ: *out = dq_tile_config(mask_id, D, dtype); return CHILL_OK;
+        case CHILL_PASS_FWD: *out = fwd_tile_config(mask_id, D, dtype, T); return CHILL_OK;
+        case CHILL_PASS_DQ: *out = dq_tile_config(mask_id, D, dtype, T); return CHILL_OK;
         case CHILL_PASS_DKDV: *out = dkdv_tile_config(mask_id, D, dtype); return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }
