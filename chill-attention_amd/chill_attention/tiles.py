@@ -15,10 +15,12 @@ from . import _lib
 _DTYPES = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}
 
 
-def tile_config(mask, head_dim: int, dtype: torch.dtype, pass_id: int, seq_len: int | None = None) -> dict:
-    """Tile shape the library uses for ``(mask class, head_dim, dtype, pass)`` on sequences of length
-    ``seq_len`` (None: the long-sequence row; the forward and dQ rows of 16-bit inputs at head dim 128
-    use a smaller workgroup for short sequences).
+def tile_config(mask, head_dim: int, dtype: torch.dtype, pass_id: int, seq_len: int | None = None,
+                batch_heads: int = 1 << 20) -> dict:
+    """Tile shape the library uses for ``(mask class, head_dim, dtype, pass)``; with ``seq_len`` (and
+    ``batch_heads`` = B * H) for a launch of that shape: the forward and dQ rows of 16-bit inputs at
+    head dim 128 use a smaller workgroup for short sequences and for grids that would not fill the chip.
+    Without ``seq_len``: the row of long sequences on a full chip.
 
     Returns ``{"rows", "streamed", "waves", "lds_bytes"}``: resident rows per workgroup (query
     rows for forward / dQ, key rows for dK/dV), rows of one streamed tile, wavefronts per
@@ -31,8 +33,8 @@ def tile_config(mask, head_dim: int, dtype: torch.dtype, pass_id: int, seq_len: 
         _lib.check("chill_tile_config", lib.chill_tile_config(mask_id, head_dim, _DTYPES[dtype], pass_id, out))
     else:
         _lib.check(
-            "chill_tile_config_for_length",
-            lib.chill_tile_config_for_length(mask_id, head_dim, _DTYPES[dtype], pass_id, seq_len, out),
+            "chill_tile_config_for_shape",
+            lib.chill_tile_config_for_shape(mask_id, head_dim, _DTYPES[dtype], pass_id, batch_heads, seq_len, out),
         )
     return {"rows": out[0], "streamed": out[1], "waves": out[2], "lds_bytes": out[3]}
 

@@ -298,12 +298,12 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
     if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
-        // the table has a row of its own for short sequences where that row differs
+        // the table has a row of its own for short sequences and small grids where that row differs
         constexpr bool has_short_row = dq_tile_config(MASK_ID, D, Elem<E>::kDType, 1).waves !=
                                        dq_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
         if constexpr (has_short_row) {
-            status = p.T <= kDqShortSequence ? launch_dq_shape<E, D, MASK_ID, true>(p, stream)
-                                             : launch_dq_shape<E, D, MASK_ID, false>(p, stream);
+            status = dq_takes_short_row((long long)p.B * p.H, p.T) ? launch_dq_shape<E, D, MASK_ID, true>(p, stream)
+                                                                   : launch_dq_shape<E, D, MASK_ID, false>(p, stream);
         } else {
             status = launch_dq_shape<E, D, MASK_ID, false>(p, stream);
         }

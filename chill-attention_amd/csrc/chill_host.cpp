@@ -118,16 +118,16 @@ int64_t chill_mask_nnz(const ChillMaskDesc* mask, int32_t T) {
 }
 
 int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int32_t out[4]) {
-    return chill_tile_config_for_length(mask_id, D, dtype, pass, kLongSequence, out);
+    return chill_tile_config_for_shape(mask_id, D, dtype, pass, 1, kLongSequence, out);
 }
 
-int chill_tile_config_for_length(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int32_t T,
-                                 int32_t out[4]) {
+int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
+                                int32_t T, int32_t out[4]) {
     if (out == nullptr) return CHILL_ERR_NULL_POINTER;
     if (!mask_id_served(mask_id)) return CHILL_ERR_BAD_MASK;
-    if (T < 1) return CHILL_ERR_BAD_ARGUMENT;
+    if (T < 1 || batch_heads < 1) return CHILL_ERR_BAD_ARGUMENT;
     TileConfig c;
-    int st = tile_config(mask_id, D, dtype, pass, T, &c);
+    int st = tile_config(mask_id, D, dtype, pass, batch_heads, T, &c);
     if (st != CHILL_OK) return st;
     out[0] = c.rows;
     out[1] = c.streamed;

@@ -66,6 +66,15 @@ constexpr bool mask_is_banded(int mask_id) {
 constexpr int kLongSequence = 0x7fffffff;
 constexpr int kFwdShortSequence = 1024;
 constexpr int kDqShortSequence = 4096;
+// The same shape is taken when the 8-wave one would leave CUs without a workgroup (B1 H8 T8192 causal:
+// forward -7 %, dQ -17 %; with twice as many heads the 8-wave shape wins again).
+constexpr int kComputeUnits = 256;
+constexpr bool fwd_takes_short_row(long long batch_heads, int T) {
+    return T <= kFwdShortSequence || batch_heads * ((T + 255) / 256) <= kComputeUnits;
+}
+constexpr bool dq_takes_short_row(long long batch_heads, int T) {
+    return T <= kDqShortSequence || batch_heads * ((T + 255) / 256) <= kComputeUnits;
+}
 
 // Forward.  16-bit inputs at head dim 128: 8 waves (256 query rows), streamed tiles of 128 keys (half
 // the barriers per key); banded masks, head dims <= 64 and short sequences: 4 waves, 64 keys, 2
@@ -192,14 +201,18 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
     return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
 }
 
-// T = sequence length the launch is for (the forward and dQ rows depend on it), kLongSequence for the
-// long-sequence row.
-inline int tile_config(int mask_id, int D, int dtype, int pass, int T, TileConfig* out) {
+// batch_heads = B * H and T = sequence length of the launch (the forward and dQ rows depend on them);
+// T = kLongSequence for the row of long sequences on a full chip.
+inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_heads, int T, TileConfig* out) {
     if (dtype != CHILL_F32 && dtype != CHILL_F16 && dtype != CHILL_BF16) return CHILL_ERR_BAD_DTYPE;
     if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
     switch (pass) {
-        case CHILL_PASS_FWD: *out = fwd_tile_config(mask_id, D, dtype, T); return CHILL_OK;
-        case CHILL_PASS_DQ: *out = dq_tile_config(mask_id, D, dtype, T); return CHILL_OK;
+        case CHILL_PASS_FWD:
+            *out = fwd_tile_config(mask_id, D, dtype, (T != kLongSequence && fwd_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
+            return CHILL_OK;
+        case CHILL_PASS_DQ:
+            *out = dq_tile_config(mask_id, D, dtype, (T != kLongSequence && dq_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
+            return CHILL_OK;
         case CHILL_PASS_DKDV: *out = dkdv_tile_config(mask_id, D, dtype); return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }

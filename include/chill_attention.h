@@ -181,12 +181,12 @@ int chill_mask_has_full_blocks(const ChillMaskDesc* mask, int32_t tile_q, int32_
  * waves_per_workgroup, lds_bytes} for (mask id, head dim, dtype, pass). */
 int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int32_t out[4]);
 
-/* The same for a launch over sequences of length T: the forward and dQ rows of 16-bit inputs at head dim
- * 128 use a smaller workgroup for short sequences (the reference's tables, autotune.py:11-119, do not
- * depend on the length; its autotuner's key does, autotune.py:129-240).  chill_tile_config reports the
- * long-sequence row. */
-int chill_tile_config_for_length(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int32_t T,
-                                 int32_t out[4]);
+/* The same for one launch, batch_heads = B * H sequences of length T: at head dim 128 the forward and dQ
+ * rows of 16-bit inputs use a smaller workgroup for short sequences and for grids that would not fill
+ * the chip (the reference's tables, autotune.py:11-119, do not depend on the shape; its autotuner's key
+ * does, autotune.py:129-240).  chill_tile_config reports the row of long sequences on a full chip. */
+int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
+                                int32_t T, int32_t out[4]);
 
 /* Number of unmasked (q, k) pairs with q, k < T, closed form per mask — the numerator of the
  * effective-FLOP metric (benchmark/benchmark.py:271-276 takes it from the dense mask). */

@@ -124,12 +124,13 @@ def test_tile_table():
         assert c["waves"] == waves, (p, D, c)
         if waves == 4:
             assert c["streamed"] == 64 and 2 * c["lds_bytes"] <= 160 * 1024
-    # short sequences at head dim 128: the 4-wave shape in forward (T <= 1024) and dQ (T <= 4096)
-    for p, T, waves in ((_lib.PASS_FWD, 1024, 4), (_lib.PASS_FWD, 1025, 8), (_lib.PASS_DQ, 4096, 4), (_lib.PASS_DQ, 4097, 8),
-                        (_lib.PASS_DKDV, 128, 8)):
-        assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T)["waves"] == waves, (p, T)
+    # short sequences and small grids at head dim 128: the 4-wave shape in forward (T <= 1024) and dQ (T <= 4096)
+    for p, T, bh, waves in ((_lib.PASS_FWD, 1024, 128, 4), (_lib.PASS_FWD, 1025, 128, 8), (_lib.PASS_DQ, 4096, 128, 4),
+                            (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_FWD, 8192, 8, 4), (_lib.PASS_FWD, 8192, 16, 8),
+                            (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 128, 8, 8)):
+        assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
-    assert _lib.lib.chill_tile_config_for_length(1, 128, _lib.BF16, 0, 0, (ctypes.c_int32 * 4)()) == -8
+    assert _lib.lib.chill_tile_config_for_shape(1, 128, _lib.BF16, 0, 1, 0, (ctypes.c_int32 * 4)()) == -8
     # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU
     for D, rows, waves in ((64, 64, 4), (32, 64, 4), (128, 128, 8)):
         c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV)
