@@ -807,6 +807,39 @@ __global__ __launch_bounds__(NW * 64) void dkdv_wide_kernel(BwdParams p, int n_k
     }
 }
 
+// One (mask, tile shape): SMALL selects the table row for grids that would not fill the chip.
+template <typename E, int D, int MASK_ID, bool SMALL>
+int launch_dkdv_shape(const BwdParams& p, hipStream_t stream) {
+    constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, SMALL);
+    constexpr int CB = dkdv_regs_blocks(D, Elem<E>::kDType);
+    constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType) && CB == 0;
+    static_assert(CB > 0 ? (cfg.rows == 128 * CB && cfg.streamed == 32 && cfg.waves == 4)
+                         : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64) : (cfg.rows == cfg.waves * 32),
+                  "tile table and kernel shape disagree");
+    const int n_k_tiles = cdiv(p.T, cfg.rows);
+    const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
+    if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
+    const int total = (int)total64;
+    dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
+    static_assert(!paired || cfg.lds_bytes >= dkdv_paired_exchange_bytes(D) * cfg.waves / 8, "LDS for the pair exchange");
+    void (*kern)(BwdParams, int, int, int);
+    if constexpr (CB > 0)
+        kern = dkdv_regs_kernel<E, D, MASK_ID, CB, dkdv_regs_stages(D)>;
+    else if constexpr (paired)
+        kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, 2>;
+    else
+        kern = dkdv_wide_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, dkdv_wide_stages(cfg.streamed, D, Elem<E>::kDType)>;
+    // mask rule order is (q tile, k tile): the streamed tile is the q tile here
+    const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, CB > 0 ? 32 * CB : 32, p.T, p.margs);
+    if (cfg.lds_bytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                cfg.lds_bytes) != hipSuccess)
+            return CHILL_ERR_HIP;
+    }
+    hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_k_tiles, total, hfb ? 1 : 0);
+    return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+}
+
 template <typename E, int D>
 int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
     int64_t max_stride = p.sq.t > p.sdo.t ? p.sq.t : p.sdo.t;
@@ -815,33 +848,15 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
     if (max_stride * Elem<E>::kBytes * 256 >= ((int64_t)1 << 31)) return CHILL_ERR_TOO_LARGE;
     int status = CHILL_ERR_BAD_MASK;
     CHILL_DISPATCH_MASK(mask_id, {
-        constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType);
-        constexpr int CB = dkdv_regs_blocks(D, Elem<E>::kDType);
-        constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType) && CB == 0;
-        static_assert(CB > 0 ? (cfg.rows == 128 * CB && cfg.streamed == 32 && cfg.waves == 4) : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64) : (cfg.rows == cfg.waves * 32),
-                      "tile table and kernel shape disagree");
-        const int n_k_tiles = cdiv(p.T, cfg.rows);
-        const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
-        if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
-        const int total = (int)total64;
-        dim3 grid(cdiv(total, 8) * 8), block(cfg.waves * 64);
-        static_assert(!paired || cfg.lds_bytes >= dkdv_paired_exchange_bytes(D) * cfg.waves / 8, "LDS for the pair exchange");
-        void (*kern)(BwdParams, int, int, int);
-        if constexpr (CB > 0)
-            kern = dkdv_regs_kernel<E, D, MASK_ID, CB, dkdv_regs_stages(D)>;
-        else if constexpr (paired)
-            kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, 2>;
-        else
-            kern = dkdv_wide_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, dkdv_wide_stages(cfg.streamed, D, Elem<E>::kDType)>;
-        // mask rule order is (q tile, k tile): the streamed tile is the q tile here
-        const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, CB > 0 ? 32 * CB : 32, p.T, p.margs);
-        if (cfg.lds_bytes > 48 * 1024) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) != hipSuccess)
-                return CHILL_ERR_HIP;
+        // the table has a row of its own for small grids where that row differs
+        constexpr bool has_small_row = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, true).waves !=
+                                       dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, false).waves;
+        if constexpr (has_small_row) {
+            status = dkdv_takes_small_row((long long)p.B * p.H_kv, p.T) ? launch_dkdv_shape<E, D, MASK_ID, true>(p, stream)
+                                                                        : launch_dkdv_shape<E, D, MASK_ID, false>(p, stream);
+        } else {
+            status = launch_dkdv_shape<E, D, MASK_ID, false>(p, stream);
         }
-        hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_k_tiles, total, hfb ? 1 : 0);
-        status = (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
     });
     return status;
 }

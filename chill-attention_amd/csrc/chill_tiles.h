@@ -156,10 +156,15 @@ constexpr bool dkdv_is_paired(int D, int dtype) { return D * elem_bytes(dtype) <
 // (measured: sliding window dK/dV -32 %, prefix-LM at D = 64 -17 %).  At D = 128 the two-stage ring of
 // such a workgroup takes 99 KiB; with a one-stage ring it fits twice but runs 8 % slower than the
 // 8-wave workgroup.
-constexpr int dkdv_paired_waves(int mask_id, int D, int dtype) {
+// `small_grid`: the 8-wave grid would cover at most half of the CUs (dkdv_takes_small_row); then the
+// 64-row workgroup is taken at every 16-bit head dim (B1 H8 T2048 D128: -17 %).
+constexpr int dkdv_paired_waves(int mask_id, int D, int dtype, bool small_grid = false) {
     (void)mask_id;
     if (CHILL_TUNE_DKDV_WAVES) return CHILL_TUNE_DKDV_WAVES;
-    return (dtype != CHILL_F32 && D <= 64) ? 4 : 8;
+    return (dtype != CHILL_F32 && (D <= 64 || small_grid)) ? 4 : 8;
+}
+constexpr bool dkdv_takes_small_row(long long batch_kv_heads, int T) {
+    return batch_kv_heads * ((T + 127) / 128) <= kComputeUnits / 2;
 }
 // at the end the waves of a pair exchange one fp32 accumulator each through LDS: 8 waves x (D rounded
 // up to 32) x 32 floats
@@ -185,14 +190,14 @@ constexpr int dkdv_regs_blocks(int D, int dtype) {
 }
 constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
 
-constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype) {
+constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype, bool small_grid = false) {
     const int row_bytes = D * elem_bytes(dtype);
     if (dkdv_regs_blocks(D, dtype) > 0) {
         const int rows = 4 * 32 * dkdv_regs_blocks(D, dtype);
         return TileConfig{rows, 32, 4, rows * row_bytes + dkdv_regs_stages(D) * (2 * 32 * row_bytes + 2 * 32 * 4)};
     }
     if (dkdv_is_paired(D, dtype)) {
-        const int waves = dkdv_paired_waves(mask_id, D, dtype);
+        const int waves = dkdv_paired_waves(mask_id, D, dtype, small_grid);
         const int rows = 16 * waves;
         const int ring = 2 * rows * row_bytes + 2 * (2 * 64 * row_bytes + 2 * 64 * 4);
         const int exchange = dkdv_paired_exchange_bytes(D) * waves / 8;
@@ -213,7 +218,10 @@ inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_
         case CHILL_PASS_DQ:
             *out = dq_tile_config(mask_id, D, dtype, (T != kLongSequence && dq_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
             return CHILL_OK;
-        case CHILL_PASS_DKDV: *out = dkdv_tile_config(mask_id, D, dtype); return CHILL_OK;
+        case CHILL_PASS_DKDV:
+            // (for this pass batch_heads counts the key / value heads)
+            *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T));
+            return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }
 }

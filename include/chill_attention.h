@@ -184,7 +184,9 @@ int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, i
 /* The same for one launch, batch_heads = B * H sequences of length T: at head dim 128 the forward and dQ
  * rows of 16-bit inputs use a smaller workgroup for short sequences and for grids that would not fill
  * the chip (the reference's tables, autotune.py:11-119, do not depend on the shape; its autotuner's key
- * does, autotune.py:129-240).  chill_tile_config reports the row of long sequences on a full chip. */
+ * does, autotune.py:129-240), and the dK/dV row one that covers half as many key rows for such grids
+ * (batch_heads = B * H_kv for that pass).  chill_tile_config reports the row of long sequences on a
+ * full chip. */
 int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
                                 int32_t T, int32_t out[4]);
 

@@ -127,7 +127,7 @@ def test_tile_table():
     # short sequences and small grids at head dim 128: the 4-wave shape in forward (T <= 1024) and dQ (T <= 4096)
     for p, T, bh, waves in ((_lib.PASS_FWD, 1024, 128, 4), (_lib.PASS_FWD, 1025, 128, 8), (_lib.PASS_DQ, 4096, 128, 4),
                             (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_FWD, 8192, 8, 4), (_lib.PASS_FWD, 8192, 16, 8),
-                            (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 128, 8, 8)):
+                            (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 2048, 8, 4), (_lib.PASS_DKDV, 2048, 16, 8)):
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
     assert _lib.lib.chill_tile_config_for_shape(1, 128, _lib.BF16, 0, 1, 0, (ctypes.c_int32 * 4)()) == -8
