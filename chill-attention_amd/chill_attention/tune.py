@@ -120,7 +120,7 @@ def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | No
     for line in text.splitlines():
         m = re.match(r"^(_ZN5chill\w+):", line)
         if m:
-            cur = m.group(1) if "_regs_kernel" in m.group(1) else None
+            cur = m.group(1) if re.search(r"_regs\d*_kernel", m.group(1)) else None
             if cur:
                 rows[cur] = {"compiler": -1, "hand": 1 << 30}
             continue
