@@ -220,45 +220,132 @@ void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
     for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(qf.c[j]), "v"(dof.c[j]));
     asm volatile("" ::"v"(lse_q), "v"(delta_q));
 
-    int st_cur = NS - 1;
-    int st_issue = LA;
-    for (int i = 0; i < n_tiles; i++) {
-        wait_async_tiles();
-        __syncthreads();
-        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
-        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
-        if (i + LA + 1 < n_tiles) issue_tile(i + LA + 1, st_issue);
-        if (i < ta || i >= tb) continue;
-        const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
-        const bool full = (i >= fa) && (i < fb);
-        const int k0 = (wg.start + i) * TK;
-        // Masked entries get a score of -inf (times the sign of the scale) in a branch of their own, so that
-        // the rest of the tile is the same straight-line code for full and partial tiles, in which the
-        // compiler places the vector work of one 32-key step among the MFMAs of the next.
+    typedef LdsTile<E, D> L;
+    constexpr bool kFold = L::kBlockAffine && Elem<E>::k16;
+    if constexpr (kFold) {
+        // Block-affine 16-bit tiles: the loop is unrolled over the ring stages and every LDS read is a
+        // loop-invariant per-lane pointer plus a constant in the instruction's offset field.  S^T and dP^T
+        // of a 32-key step are one chain of 2 NJ MFMAs whose operands are read kPrefetch steps ahead, in
+        // this order and no other (left to itself the compiler reads each operand right before its MFMA
+        // and the wave waits out the LDS latency 2 NJ times per step); the exponentials are spread over
+        // the dP^T half of the chain.
+        constexpr int kPrefetch = 4;  // C3: 2.95 ms in the compiler's order, 2.80 with 3 (then 2.84 -> 2.79 with delta in the
+                                      // accumulators, 2.76 with 4)
+        OperandPointers<E, D> at;
+        at.template init<true>(ofs, lds0);
+        // dP^T - delta comes out of the MFMA chain itself: its accumulators start at -delta (the lane's
+        // query row has one delta), which saves a subtraction per entry
+        f32x16 neg_delta;
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++) {
-            f32x16 cs, cdp;
-            gemms(cs, cdp, stage, kb);
-            if (!full) {
-                if constexpr (Mask<MASK>::kRowIsRange) {
-                    fill_outside_range(cs, vis.lo, vis.hi, k0 + 32 * kb + 4 * h, masked_score);
-                } else {
+        for (int r = 0; r < 16; r++) neg_delta[r] = -delta_q;
+        asm volatile("" : "+v"(neg_delta));
+        auto tile_step = [&](auto st_tag, int i) {
+            constexpr int ST = decltype(st_tag)::value;
+            wait_async_tiles();
+            __syncthreads();
+            if (i + LA + 1 < n_tiles) issue_tile(i + LA + 1, (ST + NS - 1) % NS);
+            if (i < ta || i >= tb) return;
+            const bool full = (i >= fa) && (i < fb);
+            const int k0 = (wg.start + i) * TK;
+            static_for<KB>([&](auto kb) {
+                constexpr int K_AT = ST * STAGE_BYTES + kb * L::BLOCK_BYTES, V_AT = K_AT + TILE_BYTES;
+                f32x16 cs, cdp;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
-                        const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
-                        cs[r] = ok ? cs[r] : masked_score;
+                for (int r = 0; r < 16; r++) {
+                    cs[r] = 0.f;
+                    cdp[r] = neg_delta[r];
+                }
+                i32x4 op[2 * NJ];
+                auto fetch = [&](auto t_tag) {
+                    constexpr int t = decltype(t_tag)::value;
+                    if constexpr (t < NJ) {
+                        op[t] = at.row_chunk(K_AT, t);
+                    } else if constexpr (t < 2 * NJ) {
+                        op[t] = at.row_chunk(V_AT, t - NJ);
+                    }
+                };
+                static_for<kPrefetch>([&](auto t) { fetch(t); });
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<NJ>([&](auto t) {
+                    cs = Elem<E>::mma(op[t], qf.c[t], cs);
+                    asm volatile("" : "+v"(cs));  // keeps the MFMA at this place of the chain
+                    fetch(std::integral_constant<int, t + kPrefetch>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                if (!full) {
+                    if constexpr (Mask<MASK>::kRowIsRange) {
+                        fill_outside_range(cs, vis.lo, vis.hi, k0 + 32 * kb + 4 * h, masked_score);
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+                            const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
+                            cs[r] = ok ? cs[r] : masked_score;
+                        }
                     }
                 }
-            }
+                constexpr int PER = (16 + NJ - 1) / NJ;  // exponentials per step
+                static_for<NJ>([&](auto t) {
+                    cdp = Elem<E>::mma(op[NJ + t], dof.c[t], cdp);
+                    asm volatile("" : "+v"(cdp));
+                    fetch(std::integral_constant<int, NJ + t + kPrefetch>{});
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float pv = fast_exp2(__builtin_fmaf(cs[r], scale, -lse_q));
-                cdp[r] = pv * (cdp[r] - delta_q);
+                    for (int r = PER * t; r < PER * (t + 1) && r < 16; r++)
+                        cs[r] = fast_exp2(__builtin_fmaf(cs[r], scale, -lse_q));
+                    // the last steps stay open to what follows: the first operands of dQ^T are read behind them
+                    if constexpr (t + 2 < NJ) __builtin_amdgcn_sched_barrier(0);
+                });
+#pragma unroll
+                for (int r = 0; r < 16; r++) cdp[r] = cs[r] * cdp[r];
+                mma_transposed<E, D>(K_AT, at, cdp, dq);  // dQ^T += K^T dS^T
+            });
+        };
+        for (int i = 0; i < n_tiles; i += NS)
+            static_for<NS>([&](auto st) {
+                if (i + st < n_tiles) tile_step(st, i + st);
+            });
+    } else {
+        int st_cur = NS - 1;
+        int st_issue = LA;
+        for (int i = 0; i < n_tiles; i++) {
+            wait_async_tiles();
+            __syncthreads();
+            st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+            st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+            if (i + LA + 1 < n_tiles) issue_tile(i + LA + 1, st_issue);
+            if (i < ta || i >= tb) continue;
+            const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
+            const bool full = (i >= fa) && (i < fb);
+            const int k0 = (wg.start + i) * TK;
+            // Masked entries get a score of -inf (times the sign of the scale) in a branch of their own, so that
+            // the rest of the tile is the same straight-line code for full and partial tiles, in which the
+            // compiler places the vector work of one 32-key step among the MFMAs of the next.
+    #pragma unroll
+            for (int kb = 0; kb < KB; kb++) {
+                f32x16 cs, cdp;
+                gemms(cs, cdp, stage, kb);
+                if (!full) {
+                    if constexpr (Mask<MASK>::kRowIsRange) {
+                        fill_outside_range(cs, vis.lo, vis.hi, k0 + 32 * kb + 4 * h, masked_score);
+                    } else {
+    #pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int k = k0 + 32 * kb + 8 * (r / 4) + 4 * h + (r % 4);
+                            const bool ok = (q_pos < seq_len) && (k < seq_len) && Mask<MASK>::pred(q_pos, k, seq_len, p.margs);
+                            cs[r] = ok ? cs[r] : masked_score;
+                        }
+                    }
+                }
+    #pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float pv = fast_exp2(__builtin_fmaf(cs[r], scale, -lse_q));
+                    cdp[r] = pv * (cdp[r] - delta_q);
+                }
+                // dQ^T += K^T dS^T
+                mma_transposed<E, D>(stage, kb, ofs, cdp, dq, lane);
             }
-            // dQ^T += K^T dS^T
-            mma_transposed<E, D>(stage, kb, ofs, cdp, dq, lane);
         }
+
     }
 
     if (q_pos < p.T)
@@ -473,25 +560,39 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
     const lds_char* k_tile = lds0;
     const lds_char* v_tile = lds0 + KV_BYTES;
 
-    int st_cur = NS - 1;
+    // Operand addresses.  Where a tile's 32-row blocks are affine, everything wave-dependent (the key
+    // block, the half of the streamed tile, the ring's place behind K and V) goes into per-lane pointers
+    // once, and the loop is unrolled over the two ring stages: every LDS read of the loop then is a
+    // loop-invariant register plus a constant in the instruction's offset field.
+    constexpr bool kFold = L::kBlockAffine && Elem<E>::k16;
+    constexpr int kPrefetch = 2;  // operand pairs read ahead in the S / dP chain (C3: 4.05 ms in the compiler's order, 3.92 with 2, 3.98 with 3)
+    OperandPointers<E, D> at_k, at_q;  // K / V rows of this wave's key block; Q / dO rows of its half
+    const lds_char* vec0 = lds0 + RING_OFF + 2 * TILE_BYTES + (32 * half + 4 * h) * 4;  // LSE2 / delta of the lane's 16 rows
+    if constexpr (kFold) {
+        at_k.template init<false>(ofs, lds0 + kblk * L::BLOCK_BYTES);
+        at_q.template init<true>(ofs, lds0 + RING_OFF + half * L::BLOCK_BYTES);
+        asm volatile("" : "+v"(vec0));
+    }
+
     int tile = -1;  // position of iteration `it` inside the q-tile range (it % n_tiles)
-    for (int it = 0; it < n_iters; it++) {
+    // iteration `it` consumes ring stage ST = it % 2
+    auto iteration = [&](auto st_tag, int it) {
+        constexpr int ST = decltype(st_tag)::value;
         wait_async_tiles();
         __syncthreads();
-        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
         tile = tile + 1 == n_tiles ? 0 : tile + 1;
-        const int st_next = st_cur + 1 == NS ? 0 : st_cur + 1;
         const bool in_block = !(tile < ta || tile >= tb);
         // the two waves that share a SIMD issue their loads at different points of the iteration, so
         // that one of them keeps the matrix pipe busy while the other sits in the memory pipeline
         const bool issue_late = in_block && half == 1;
         if (!issue_late) {
-            if (it + 1 < n_iters) issue_next(st_next);
+            if (it + 1 < n_iters) issue_next(1 - ST);
         }
-        if (!in_block) continue;
-        const lds_char* q_tile = lds0 + RING_OFF + st_cur * STAGE_BYTES;
+        if (!in_block) return;
+        const lds_char* q_tile = lds0 + RING_OFF + ST * STAGE_BYTES;
         const lds_char* do_tile = q_tile + TILE_BYTES;
-        const lds_float* vec = reinterpret_cast<const lds_float*>(q_tile + 2 * TILE_BYTES) + 32 * half;
+        const lds_char* vec = vec0 + ST * STAGE_BYTES;
+        constexpr int Q_AT = ST * STAGE_BYTES, DO_AT = Q_AT + TILE_BYTES;
         const bool full = (tile >= fa) && (tile < fb);
         const int q0 = (wg.start + tile) * TQS + 32 * half;
 
@@ -501,20 +602,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
         // Masked entries get a score of -inf (times the sign of the scale) in a branch of their own, so
         // that the rest of the block is the same straight-line code for full and partial tiles.
         f32x4 lse4[4], del4[4];
+        auto read_lse = [&]() {
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++)
-            lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h);
+            for (int g4 = 0; g4 < 4; g4++)
+                lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 32 * g4);
+        };
+        if constexpr (!(kFold && kPrefetch > 0)) read_lse();
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             s[r] = 0.f;
             dp[r] = 0.f;
         }
-#pragma unroll
-        for (int j = 0; j < NJ; j++) {
-            s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
-        }
-        if (!full) {
+        auto mask_scores = [&]() {
             if constexpr (Mask<MASK>::kRowIsRange) {
                 fill_outside_range(s, vis.lo, vis.hi, q0 + 4 * h, masked_score);
             } else {
@@ -531,22 +631,89 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
                 const float l = lse4[r / 4][r % 4];
                 lse4[r / 4][r % 4] = (l == -INFINITY) ? 0.f : l;
             }
+        };
+        if constexpr (kFold && kPrefetch > 0) {
+            // S = Q K^T and dP = dO V^T as one chain of 2 NJ MFMAs whose operand pairs are read kPrefetch
+            // steps ahead, in this order and no other: left to itself the compiler reads each pair right
+            // before its MFMA, and the wave waits out the LDS latency 2 NJ times per block.  The
+            // exponentials of S are spread over the dP half of the chain.
+            i32x4 opa[2 * NJ], opb[2 * NJ];
+            auto fetch = [&](auto t_tag) {
+                constexpr int t = decltype(t_tag)::value;
+                if constexpr (t < NJ) {
+                    opa[t] = at_q.row_chunk(Q_AT, t);
+                    opb[t] = at_k.row_chunk(0, t);
+                } else if constexpr (t < 2 * NJ) {
+                    opa[t] = at_q.row_chunk(DO_AT, t - NJ);
+                    opb[t] = at_k.row_chunk(KV_BYTES, t - NJ);
+                }
+            };
+            static_for<kPrefetch>([&](auto t) { fetch(t); });
+            __builtin_amdgcn_sched_barrier(0);
+            static_for<NJ>([&](auto t) {
+                s = Elem<E>::mma(opa[t], opb[t], s);
+                asm volatile("" : "+v"(s));  // keeps the MFMA at this place of the chain
+                fetch(std::integral_constant<int, t + kPrefetch>{});
+                if constexpr (t == NJ / 2) read_lse();  // needed from the first step of the dP half on
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if (!full) mask_scores();
+            constexpr int PER = (16 + NJ - 1) / NJ;  // exponentials per step
+            static_for<NJ>([&](auto t) {
+                dp = Elem<E>::mma(opa[NJ + t], opb[NJ + t], dp);
+                asm volatile("" : "+v"(dp));  // keeps the MFMA at this place of the chain
+                fetch(std::integral_constant<int, NJ + t + kPrefetch>{});
+#pragma unroll
+                for (int r = PER * t; r < PER * (t + 1) && r < 16; r++)
+                    s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
+                // the last steps stay open to what follows: the first operands of dV^T are read behind them
+                if constexpr (t + 2 < NJ) __builtin_amdgcn_sched_barrier(0);
+            });
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                if constexpr (kFold) {
+                    s = Elem<E>::mma(at_q.row_chunk(Q_AT, j), at_k.row_chunk(0, j), s);
+                } else {
+                    s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
+                }
+            }
+            if (!full) mask_scores();
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                if constexpr (kFold) {
+                    dp = Elem<E>::mma(at_q.row_chunk(DO_AT, j), at_k.row_chunk(KV_BYTES, j), dp);
+                } else {
+                    dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
         }
 #pragma unroll
-        for (int j = 0; j < NJ; j++)
-            dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
-#pragma unroll
         for (int g4 = 0; g4 < 4; g4++)
-            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 8 * g4 + 4 * h);
-        mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);  // dV^T += dO^T P
+            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + VEC_BYTES + 32 * g4);
+        // dV^T += dO^T P
+        if constexpr (kFold) {
+            mma_transposed<E, D>(DO_AT, at_q, s, dv);
+        } else {
+            mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);
+        }
         if (issue_late) {
-            if (it + 1 < n_iters) issue_next(st_next);
+            if (it + 1 < n_iters) issue_next(1 - ST);
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) dp[r] = s[r] * (dp[r] - del4[r / 4][r % 4]);
-        mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);  // dK^T += Q^T dS
+        // dK^T += Q^T dS
+        if constexpr (kFold) {
+            mma_transposed<E, D>(Q_AT, at_q, dp, dk);
+        } else {
+            mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);
+        }
+    };
+    for (int it = 0; it < n_iters; it += 2) {
+        iteration(std::integral_constant<int, 0>{}, it);
+        if (it + 1 < n_iters) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
 
     // Sum the two waves of a pair through LDS and store: the waves of the second half hand their dK^T

@@ -576,6 +576,52 @@ struct OperandOffsets {
     }
 };
 
+// The same operands through per-lane POINTERS that already include everything wave-dependent (the
+// LDS base, the wave's 32-row block of a tile, a region's place in LDS): what a use adds is a
+// compile-time constant, which goes into the offset field of the LDS instruction, so a loop over tiles
+// at fixed places spends no vector instruction on addresses.  The pointers pass through an empty asm:
+// the compiler keeps them in registers instead of re-deriving them at every use.  Block-affine 16-bit
+// tiles only; offsets must stay below 64 KiB.
+template <typename E, int D>
+struct OperandPointers {
+    typedef LdsTile<E, D> L;
+    typedef OperandOffsets<E, D> O;
+    const lds_char* row[O::NJ];
+    const lds_char* tr[O::DB][O::NS_TR][2];
+
+    template <bool WITH_TR>
+    __device__ __forceinline__ void init(const O& ofs, const lds_char* base) {
+        static_assert(L::kBlockAffine && Elem<E>::k16, "block-affine 16-bit tiles");
+#pragma unroll
+        for (int j = 0; j < O::NJ; j++) {
+            row[j] = base + ofs.row[j];
+            asm volatile("" : "+v"(row[j]));
+        }
+        if constexpr (WITH_TR) {
+#pragma unroll
+            for (int db = 0; db < O::DB; db++)
+#pragma unroll
+                for (int s = 0; s < O::NS_TR; s++)
+#pragma unroll
+                    for (int w = 0; w < 2; w++) {
+                        tr[db][s][w] = base + ofs.tr[db][s][w];
+                        asm volatile("" : "+v"(tr[db][s][w]));
+                    }
+        }
+    }
+    // rows 0..31 of the tile `imm` bytes behind the base
+    __device__ __forceinline__ i32x4 row_chunk(int imm, int j) const {
+        return *reinterpret_cast<const lds_i32x4*>(row[j] + imm);
+    }
+    __device__ __forceinline__ i32x4 tr_operand(int imm, int s, int db) const {
+        const int at = imm + (O::kHalfAffine ? s * 16 * O::ROW_BYTES : 0);
+        i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(tr[db][O::kHalfAffine ? 0 : s][0] + at));
+        i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(tr[db][O::kHalfAffine ? 0 : s][1] + at));
+        i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(i32x4, v);
+    }
+};
+
 // acc(32 rows of the LDS tile x 32 cols) += X[32*kb + 0..31][:] * B^T, B = resident rows.
 template <typename E, int D>
 __device__ __forceinline__ f32x16 mma_rowwise(const lds_char* tile, int kb, const OperandOffsets<E, D>& ofs,
@@ -629,6 +675,22 @@ __device__ __forceinline__ void mma_transposed(const lds_char* tile, int kb, con
                 acc[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, p[r], acc[db], 0, 0, 0);
             }
         }
+    }
+}
+
+// acc^T += X^T P with X the 32 rows behind the pointers (see OperandPointers)
+template <typename E, int D>
+__device__ __forceinline__ void mma_transposed(int imm, const OperandPointers<E, D>& ptrs, const f32x16& p,
+                                               f32x16 (&acc)[(D + 31) / 32]) {
+    constexpr int DB = (D + 31) / 32;
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        f32x8 ps;
+#pragma unroll
+        for (int e = 0; e < 8; e++) ps[e] = p[8 * s + e];
+        const i32x4 bop = Elem<E>::pack8(ps);
+#pragma unroll
+        for (int db = 0; db < DB; db++) acc[db] = Elem<E>::mma(ptrs.tr_operand(imm, s, db), bop, acc[db]);
     }
 }
 
