@@ -565,7 +565,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
     // once, and the loop is unrolled over the two ring stages: every LDS read of the loop then is a
     // loop-invariant register plus a constant in the instruction's offset field.
     constexpr bool kFold = L::kBlockAffine && Elem<E>::k16;
-    constexpr int kPrefetch = 2;  // operand pairs read ahead in the S / dP chain (C3: 4.05 ms in the compiler's order, 3.92 with 2, 3.98 with 3)
+    // operands read ahead in a block's MFMA chain (folded path only).  C3: 4.05 ms in the compiler's order,
+    // 3.97 with the S / dP part of the chain two ahead, 3.90 with the whole chain two ahead; three ahead
+    // 3.98, the transposed operands three or four ahead 4.10 / 4.17 (more requests in flight per wave
+    // only lengthen the queue of the LDS, which is busy 45 % of the time)
+    constexpr int kPrefetch = 2 < NJ ? 2 : NJ;
+    constexpr int kPrefetchTr = kPrefetch;
+    static_assert(kPrefetchTr >= kPrefetch && kPrefetch >= 1, "read-ahead distances");
     OperandPointers<E, D> at_k, at_q;  // K / V rows of this wave's key block; Q / dO rows of its half
     const lds_char* vec0 = lds0 + RING_OFF + 2 * TILE_BYTES + (32 * half + 4 * h) * 4;  // LSE2 / delta of the lane's 16 rows
     if constexpr (kFold) {
@@ -607,7 +613,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
             for (int g4 = 0; g4 < 4; g4++)
                 lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 32 * g4);
         };
-        if constexpr (!(kFold && kPrefetch > 0)) read_lse();
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -632,83 +637,104 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
                 lse4[r / 4][r % 4] = (l == -INFINITY) ? 0.f : l;
             }
         };
-        if constexpr (kFold && kPrefetch > 0) {
-            // S = Q K^T and dP = dO V^T as one chain of 2 NJ MFMAs whose operand pairs are read kPrefetch
-            // steps ahead, in this order and no other: left to itself the compiler reads each pair right
-            // before its MFMA, and the wave waits out the LDS latency 2 NJ times per block.  The
-            // exponentials of S are spread over the dP half of the chain.
-            i32x4 opa[2 * NJ], opb[2 * NJ];
+        if constexpr (kFold) {
+            // The block's 2 NJ + 4 DB MFMAs — S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS — as one
+            // chain whose LDS operands are read kPrefetch steps ahead, in this order and no other: left to
+            // itself the compiler reads most operands right before their MFMA, and the wave waits out the
+            // LDS latency again and again.  The vector work rides along: the exponentials on the dP
+            // steps, dS on the dV^T steps.
+            constexpr int N1 = NJ, N2 = 2 * NJ, N3 = N2 + 2 * DB, N4 = N3 + 2 * DB;
+            i32x4 opa[N4], opb[N2];
             auto fetch = [&](auto t_tag) {
                 constexpr int t = decltype(t_tag)::value;
-                if constexpr (t < NJ) {
+                if constexpr (t < N1) {
                     opa[t] = at_q.row_chunk(Q_AT, t);
                     opb[t] = at_k.row_chunk(0, t);
-                } else if constexpr (t < 2 * NJ) {
-                    opa[t] = at_q.row_chunk(DO_AT, t - NJ);
-                    opb[t] = at_k.row_chunk(KV_BYTES, t - NJ);
+                } else if constexpr (t < N2) {
+                    opa[t] = at_q.row_chunk(DO_AT, t - N1);
+                    opb[t] = at_k.row_chunk(KV_BYTES, t - N1);
+                } else if constexpr (t < N3) {
+                    opa[t] = at_q.tr_operand(DO_AT, (t - N2) / DB, (t - N2) % DB);
+                } else if constexpr (t < N4) {
+                    opa[t] = at_q.tr_operand(Q_AT, (t - N3) / DB, (t - N3) % DB);
                 }
+            };
+            // operand i is read at step i - kPrefetch (row-wise pairs, 8 registers) or i - kPrefetchTr
+            // (transposed operands, 4 registers); what falls before step 0 is read up front
+            auto ahead = [&](auto t_tag) {
+                constexpr int t = decltype(t_tag)::value;
+                if constexpr (t + kPrefetch < N2) fetch(std::integral_constant<int, t + kPrefetch>{});
+                if constexpr (t + kPrefetchTr >= N2) fetch(std::integral_constant<int, t + kPrefetchTr>{});
             };
             static_for<kPrefetch>([&](auto t) { fetch(t); });
             __builtin_amdgcn_sched_barrier(0);
             static_for<NJ>([&](auto t) {
                 s = Elem<E>::mma(opa[t], opb[t], s);
                 asm volatile("" : "+v"(s));  // keeps the MFMA at this place of the chain
-                fetch(std::integral_constant<int, t + kPrefetch>{});
-                if constexpr (t == NJ / 2) read_lse();  // needed from the first step of the dP half on
+                ahead(t);
+                if constexpr (t == NJ / 2) read_lse();  // needed from the first step of the dP part on
                 __builtin_amdgcn_sched_barrier(0);
             });
             if (!full) mask_scores();
-            constexpr int PER = (16 + NJ - 1) / NJ;  // exponentials per step
+            constexpr int PER = (16 + NJ - 1) / NJ;  // exponentials per dP step
+            i32x4 pb[2], dsb[2];
             static_for<NJ>([&](auto t) {
-                dp = Elem<E>::mma(opa[NJ + t], opb[NJ + t], dp);
-                asm volatile("" : "+v"(dp));  // keeps the MFMA at this place of the chain
-                fetch(std::integral_constant<int, NJ + t + kPrefetch>{});
+                dp = Elem<E>::mma(opa[N1 + t], opb[N1 + t], dp);
+                asm volatile("" : "+v"(dp));
+                ahead(std::integral_constant<int, N1 + t>{});
 #pragma unroll
                 for (int r = PER * t; r < PER * (t + 1) && r < 16; r++)
                     s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
-                // the last steps stay open to what follows: the first operands of dV^T are read behind them
-                if constexpr (t + 2 < NJ) __builtin_amdgcn_sched_barrier(0);
+                if constexpr (t == NJ / 2) {
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; g4++)
+                        del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + VEC_BYTES + 32 * g4);
+                }
+                if constexpr (t == NJ - 1) pack_block<E>(s, pb);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            constexpr int PERD = (16 + 2 * DB - 1) / (2 * DB);  // entries of dS per dV^T step
+            static_for<2 * DB>([&](auto u) {
+                constexpr int db = u % DB;
+                dv[db] = Elem<E>::mma(opa[N2 + u], pb[u / DB], dv[db]);
+                asm volatile("" : "+v"(dv[db]));
+                ahead(std::integral_constant<int, N2 + u>{});
+#pragma unroll
+                for (int r = PERD * u; r < PERD * (u + 1) && r < 16; r++) dp[r] = s[r] * (dp[r] - del4[r / 4][r % 4]);
+                if constexpr (u == 2 * DB - 1) pack_block<E>(dp, dsb);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if (issue_late) {
+                if (it + 1 < n_iters) issue_next(1 - ST);
+            }
+            static_for<2 * DB>([&](auto u) {
+                constexpr int db = u % DB;
+                dk[db] = Elem<E>::mma(opa[N3 + u], dsb[u / DB], dk[db]);
+                asm volatile("" : "+v"(dk[db]));
+                ahead(std::integral_constant<int, N3 + u>{});
+                __builtin_amdgcn_sched_barrier(0);
             });
         } else {
+            read_lse();
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                if constexpr (kFold) {
-                    s = Elem<E>::mma(at_q.row_chunk(Q_AT, j), at_k.row_chunk(0, j), s);
-                } else {
-                    s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
-                }
-            }
+            for (int j = 0; j < NJ; j++)
+                s = Elem<E>::mma(ofs.row_chunk(q_tile, half, j, lane), ofs.row_chunk(k_tile, kblk, j, lane), s);
             if (!full) mask_scores();
 #pragma unroll
-            for (int j = 0; j < NJ; j++) {
-                if constexpr (kFold) {
-                    dp = Elem<E>::mma(at_q.row_chunk(DO_AT, j), at_k.row_chunk(KV_BYTES, j), dp);
-                } else {
-                    dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
-                }
-            }
+            for (int j = 0; j < NJ; j++)
+                dp = Elem<E>::mma(ofs.row_chunk(do_tile, half, j, lane), ofs.row_chunk(v_tile, kblk, j, lane), dp);
 #pragma unroll
             for (int r = 0; r < 16; r++) s[r] = fast_exp2(__builtin_fmaf(s[r], scale, -lse4[r / 4][r % 4]));
-        }
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++)
-            del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + VEC_BYTES + 32 * g4);
-        // dV^T += dO^T P
-        if constexpr (kFold) {
-            mma_transposed<E, D>(DO_AT, at_q, s, dv);
-        } else {
-            mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);
-        }
-        if (issue_late) {
-            if (it + 1 < n_iters) issue_next(1 - ST);
-        }
+            for (int g4 = 0; g4 < 4; g4++)
+                del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + VEC_BYTES + 32 * g4);
+            mma_transposed<E, D>(do_tile, half, ofs, s, dv, lane);  // dV^T += dO^T P
+            if (issue_late) {
+                if (it + 1 < n_iters) issue_next(1 - ST);
+            }
 #pragma unroll
-        for (int r = 0; r < 16; r++) dp[r] = s[r] * (dp[r] - del4[r / 4][r % 4]);
-        // dK^T += Q^T dS
-        if constexpr (kFold) {
-            mma_transposed<E, D>(Q_AT, at_q, dp, dk);
-        } else {
-            mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);
+            for (int r = 0; r < 16; r++) dp[r] = s[r] * (dp[r] - del4[r / 4][r % 4]);
+            mma_transposed<E, D>(q_tile, half, ofs, dp, dk, lane);  // dK^T += Q^T dS
         }
     };
     for (int it = 0; it < n_iters; it += 2) {
