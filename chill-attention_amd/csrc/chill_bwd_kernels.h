@@ -408,8 +408,9 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
 // through LDS at the end.  Splitting the QUERY axis inside a pair keeps the per-wave state (two
 // 32 x D accumulators, no resident MFMA operands) within 256 registers, so two waves share a SIMD
 // and one wave's vector work hides behind the other's MFMAs, with no redundant MFMA work.
+// Four-wave workgroups are compiled for two per CU, those of head dims <= 64 (50 KiB of LDS) for three: 168 registers.
 template <typename E, int D, int MASK, int NW, int NS>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4 ? 2 : 1))) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4 ? (D <= 64 ? 3 : 2) : 1))) void dkdv_kernel(BwdParams p, int n_k_tiles, int total_items,
                                                        int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     typedef LdsTile<E, D> L;
@@ -564,7 +565,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
     // block, the half of the streamed tile, the ring's place behind K and V) goes into per-lane pointers
     // once, and the loop is unrolled over the two ring stages: every LDS read of the loop then is a
     // loop-invariant register plus a constant in the instruction's offset field.
-    constexpr bool kFold = L::kBlockAffine && Elem<E>::k16;
+    // Not for the 4-wave workgroups of head dims <= 64: they run three to a CU at <= 168 registers, which the
+    // pointers would exceed (B4 H32 T8192 D64 causal: 2.29 ms as they are, 2.38 folded and chained, 2.46 folded only)
+    constexpr bool kFold = L::kBlockAffine && Elem<E>::k16 && (NW == 8 || D >= 128);
     // operands read ahead in a block's MFMA chain (folded path only).  C3: 4.05 ms in the compiler's order,
     // 3.97 with the S / dP part of the chain two ahead, 3.90 with the whole chain two ahead; three ahead
     // 3.98, the transposed operands three or four ahead 4.10 / 4.17 (more requests in flight per wave
