@@ -14,8 +14,14 @@
 // tile i+2 is in flight.  Work proceeds in steps of 32 keys, software-pipelined: the score MFMAs of
 // step t+1 are issued before the softmax of step t, so matrix and vector units overlap in a wave.
 //
-// The softmax rescales lazily: a row's reference max is raised (and O, l rescaled) only when a
-// block max exceeds it by more than kRescaleTau, a wave-uniform rare branch.
+// The softmax rescales lazily.  fp32 inputs: a row's reference max is raised (and O, l rescaled) only
+// when a block max exceeds it by more than kRescaleTau, a wave-uniform rare branch.  16-bit inputs
+// compute no block max at all on the common path: a row keeps the max of its first visible block as
+// reference while the block sums of P stay below a limit far inside the range of P's type (fp16:
+// 2^15, bf16: 1e18), and only a block whose sum exceeds it (or a row without reference yet) takes the
+// branch that computes the block max, raises the reference and redoes the block's P from the raw
+// scores, which are kept until then (chill_fwd.py:213-222 recomputes the max for every block; O and
+// LSE2 do not depend on the reference beyond rounding).
 //
 // Tile skipping and the predicate-free path follow chill_fwd.py:131-139 and :161-185, evaluated
 // per WAVE (32 rows): a wave skips streamed tiles outside its own k-range and drops the predicate
@@ -137,6 +143,13 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
     // A negative scale reverses the order of the scores: the sign goes into Q, the softmax works
     // with |scale| (max(scale * s) = |scale| * max(sign * s)).
     const float scale = fabsf(p.scale_log2);
+    // guarded softmax (16-bit inputs): see the step
+    // not for the banded masks: their rows end after a few blocks, of which the first always takes the branch
+    // (chunkwise fp16 T=16384 D=128: forward 0.43 ms with the guard, 0.42 without)
+    constexpr bool kGuard = Elem<E>::k16 && !mask_is_banded(MASK);
+    // a block sum below the limit keeps every P of the block inside fp16 (65504) / far inside bf16
+    constexpr float kGuardLimit = Elem<E>::kDType == CHILL_F16 ? 32768.f : 1.0e18f;
+    float guard_above = -1.f;
 
     // K operands of the score block of step kb of the tile at `stage` (rows 32*kb .. 32*kb+31),
     // read one step ahead of the MFMAs that consume them
@@ -155,20 +168,23 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
 #pragma unroll
         for (int j = 0; j < NJ; j++) dst = Elem<E>::mma(ko.c[j], qf.c[j], dst);
     };
-    // mask and block max (scaled) of a score block
-    auto prepare = [&](f32x16& sc, bool full, int key0) -> float {
-        if (!full) {
-            if constexpr (M::kRowIsRange) {
-                fill_outside_range(sc, vis.lo, vis.hi, key0 + 4 * h, -INFINITY);
-            } else {
+    // mask of a partial score block
+    auto mask_block = [&](f32x16& sc, int key0) {
+        if constexpr (M::kRowIsRange) {
+            fill_outside_range(sc, vis.lo, vis.hi, key0 + 4 * h, -INFINITY);
+        } else {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
-                    bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
-                    sc[r] = ok ? sc[r] : -INFINITY;
-                }
+            for (int r = 0; r < 16; r++) {
+                int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+                bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
+                sc[r] = ok ? sc[r] : -INFINITY;
             }
         }
+    };
+    // mask and block max (scaled) of a score block
+    auto prepare = [&](f32x16& sc, bool full, int key0) -> float {
+        if (!full) mask_block(sc, key0);
+        if constexpr (kGuard) return 0.f;
         float mx = sc[0];
 #pragma unroll
         for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
@@ -195,14 +211,19 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
         }
     };
     // O^T += V^T P^T
-    auto accumulate = [&](const f32x16& pr, const VOperands& vo, const lds_char* stage, int kb) {
+    auto accumulate = [&](const f32x16& pr, const i32x4 (&packed)[2], const VOperands& vo, const lds_char* stage, int kb) {
         if constexpr (Elem<E>::k16) {
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
-                f32x8 ps;
+                i32x4 bop;
+                if constexpr (kGuard) {
+                    bop = packed[s2];
+                } else {
+                    f32x8 ps;
 #pragma unroll
-                for (int e = 0; e < 8; e++) ps[e] = pr[8 * s2 + e];
-                const i32x4 bop = Elem<E>::pack8(ps);
+                    for (int e = 0; e < 8; e++) ps[e] = pr[8 * s2 + e];
+                    bop = Elem<E>::pack8(ps);
+                }
 #pragma unroll
                 for (int db = 0; db < DB; db++) {
                     i16x8 av = __builtin_shufflevector(vo.lo[s2][db], vo.hi[s2][db], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -244,19 +265,21 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
     auto step = [&](const lds_char* stage, const lds_char* stage_next, int kb, bool full, bool full_next, int k0) {
         f32x16& cur = s[kb & 1];
         f32x16& nxt = s[(kb + 1) & 1];
-        // rare path: raise the reference max and rescale what has been accumulated
-        const bool raise = mx_cur > m_run + kRescaleTau;
-        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-            const float m_new = raise ? mx_cur : m_run;
-            const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = fast_exp2(m_use - m_use_new);
-            m_run = m_new;
-            m_use = m_use_new;
-            l_run *= alpha;
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+        if constexpr (!kGuard) {
+            // rare path: raise the reference max and rescale what has been accumulated
+            const bool raise = mx_cur > m_run + kRescaleTau;
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+                const float m_new = raise ? mx_cur : m_run;
+                const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = fast_exp2(m_use - m_use_new);
+                m_run = m_new;
+                m_use = m_use_new;
+                l_run *= alpha;
+    #pragma unroll
+                for (int db = 0; db < DB; db++)
+    #pragma unroll
+                    for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+            }
         }
         const bool in_tile = kb + 1 < KB;
         const bool have_next = in_tile || LA >= 1;
@@ -268,11 +291,54 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
         // scores of the next step (operands already in registers) fly while this step's softmax runs
         if (have_next) scores(nxt, ka);
         float psum = 0.f;
+        i32x4 pb[2];
+        if constexpr (kGuard) {
+            // P against the reference the row has, packed at once; the raw scores stay in `cur`
+            auto softmax_block = [&]() {
+                psum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            float pv = fast_exp2(__builtin_fmaf(cur[r], scale, -m_use));
-            cur[r] = pv;
-            psum += pv;
+                for (int s2 = 0; s2 < 2; s2++) {
+                    f32x8 ps;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        ps[e] = fast_exp2(__builtin_fmaf(cur[8 * s2 + e], scale, -m_use));
+                        psum += ps[e];
+                    }
+                    pb[s2] = Elem<E>::pack8(ps);
+                }
+            };
+            softmax_block();
+            // No block max on this path.  A row takes the max of its first block with a visible key as
+            // reference and keeps it while the block sums stay below guard_above (far from the range of
+            // P's type); a row without reference has guard_above = -1 and always comes here.
+            const unsigned long long fired = __builtin_amdgcn_ballot_w64(psum > guard_above);
+            if (fired != 0) {
+                // the two lanes of a row (l and l ^ 32) hold half of its keys each and share its reference
+                const bool fire = (((fired | (fired >> 32) | (fired << 32)) >> lane) & 1) != 0;
+                float mx = cur[0];
+#pragma unroll
+                for (int r = 1; r < 16; r++) mx = fmaxf(mx, cur[r]);
+                mx = max_across_halves(mx) * scale;
+                const float m_new = fire ? fmaxf(m_run, mx) : m_run;
+                const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
+                const float alpha = fast_exp2(m_use - m_use_new);
+                m_run = m_new;
+                m_use = m_use_new;
+                guard_above = (m_new == -INFINITY) ? -1.f : kGuardLimit;
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; db++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+                softmax_block();
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float pv = fast_exp2(__builtin_fmaf(cur[r], scale, -m_use));
+                cur[r] = pv;
+                psum += pv;
+            }
         }
         l_run += psum;
         __builtin_amdgcn_sched_barrier(0);
@@ -282,8 +348,18 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
         } else if (KB > 1 && LA >= 1) {
             load_k_operands(ka, stage_next, kb + 2 - KB);
         }
-        accumulate(cur, vo, stage, kb);
-        if (have_next) mx_cur = in_tile ? prepare(nxt, full, k0 + 32 * (kb + 1)) : prepare(nxt, full_next, k0 + TK);
+        accumulate(cur, pb, vo, stage, kb);
+        if constexpr (kGuard) {
+            if (have_next) {
+                if (in_tile) {
+                    if (!full) mask_block(nxt, k0 + 32 * (kb + 1));
+                } else {
+                    if (!full_next) mask_block(nxt, k0 + TK);
+                }
+            }
+        } else {
+            if (have_next) mx_cur = in_tile ? prepare(nxt, full, k0 + 32 * (kb + 1)) : prepare(nxt, full_next, k0 + TK);
+        }
     };
 
     int st_cur = NS - 1;  // LDS stage of tile i (advanced at the top of the loop)

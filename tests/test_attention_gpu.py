@@ -142,6 +142,32 @@ def test_lse_and_fully_masked_rows():
     assert torch.equal(o3, o4)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,growth", [(torch.float16, 60.0), (torch.bfloat16, 400.0), (torch.float32, 60.0)], ids=str)
+def test_reference_max_is_raised_along_the_keys(dtype, growth):
+    """Scores that grow by `growth` (log2 units) along the key axis: the forward's reference max has to be
+    raised many times per row (16-bit inputs: whenever a block's sum of P leaves the guarded range), in rows
+    whose two half-wave lanes see different sums.  Same bar as the other forward tests."""
+    torch.manual_seed(7)
+    B, H, T, D = 1, 2, 1024, 64
+    q = torch.randn(B, H, T, D, device=DEV) * 0.5
+    k = torch.randn(B, H, T, D, device=DEV) * 0.5
+    v = torch.randn(B, H, T, D, device=DEV)
+    # a common direction whose weight in k grows with the key position: score(q, k_t) ~ t * growth / T (log2 units)
+    u = torch.nn.functional.normalize(torch.randn(D, device=DEV), dim=0)
+    q = q + 4.0 * u
+    ramp = torch.arange(T, device=DEV, dtype=torch.float32) / T
+    k = k + (growth * (D ** 0.5) / (4.0 * 1.4427)) * ramp[None, None, :, None] * u
+    q, k, v = (x.to(dtype) for x in (q, k, v))
+    for m in (MASK_INSTANCES[0], MASK_INSTANCES[1]):
+        mask = make_mask(m)
+        ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), None)
+        out, lse = ca.chill_attention(q, k, v, mask=mask, return_lse=True)
+        atol, rtol = OUT_TOL[dtype]
+        assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+        torch.testing.assert_close(out * res_mask, ref.to(dtype), atol=atol, rtol=rtol)
+
+
 def test_rows_without_keys():
     """A query whose keys are all masked (possible with lens cutting a window that only looks ahead)."""
     m = ("SlidingWindowChillMask", (0, 0))
