@@ -36,10 +36,10 @@ PEAK_HBM_GBS = 8000.0
 # the same counters read for a plain 1 GiB copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
 # the summaries of those runs are kept under profiles/.  (workload, kernel) -> bytes
 MEASURED_TRAFFIC = {
-    ("C3", "chill_fwd"): (710245 * 2.0 + 266243) * 1024,
-    ("C3", "chill_bwd_delta"): (262171 * 2.0 + 4197) * 1024,
-    ("C3", "chill_bwd_dkdv"): (548889 * 2.0 + 540259) * 1024,
-    ("C3", "chill_bwd_dq"): (756268 * 2.0 + 262144) * 1024,
+    ("C3", "chill_fwd"): (696510 * 2.0 + 266243) * 1024,
+    ("C3", "chill_bwd_delta"): (262171 * 2.0 + 4193) * 1024,
+    ("C3", "chill_bwd_dkdv"): (534807 * 2.0 + 540102) * 1024,
+    ("C3", "chill_bwd_dq"): (747358 * 2.0 + 262144) * 1024,
 }
 
 # name -> (mask ctor name, args, dtype, B, H, T, D, seed, sigma)
