@@ -29,6 +29,9 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
                                                 int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     using M = Mask<MASK>;
+    // guarded softmax (see fwd_kernel): not for the banded masks, whose rows end after a few blocks
+    constexpr bool kGuard = !mask_is_banded(MASK);
+    constexpr float kGuardLimit = Elem<E>::kDType == CHILL_F16 ? 32768.f : 1.0e18f;
     static_assert(Elem<E>::k16, "16-bit element types");
     typedef FwdLds<E, D, TK> Lds;
     typedef typename Lds::KT KT;
@@ -143,16 +146,15 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
                 }
             }
         }
+        if constexpr (kGuard) return 0.f;  // no block max on the common path
         float mx = sc[0];
 #pragma unroll
         for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
         return max_across_halves(mx) * scale;
     };
     // O^T += V^T P^T for step kb: one packed P operand per 16 keys feeds all head-dim blocks
-    auto accumulate = [&](const f32x16& pr, const lds_char* stage, int kb) {
+    auto accumulate = [&](const i32x4 (&bop)[2], const lds_char* stage, int kb) {
         const lds_char* base = stage + v_lane + kb * 32 * VT::PITCH;
-        i32x4 bop[2];
-        pack_block<E>(pr, bop);
         static_for<2>([&](auto s2) {
             static_for<DB>([&](auto db) {
                 const lds_char* a0 = base + (16 * s2) * VT::PITCH + db * 64;
@@ -166,6 +168,7 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
 
     f32x16 s[2];         // scores of the current and of the next step
     float mx_cur = 0.f;  // block max of s[current], already scaled
+    float guard_above = -1.f;
     const lds_char* lds0 = (const lds_char*)smem;
     // Q must have arrived before the loop: inside it the only vector-memory traffic is the async
     // tile loads, and the compiler must not place a wait for them in front of the first MFMA
@@ -183,12 +186,11 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
     auto step = [&](const lds_char* stage, int kb, bool full, int k0) {
         f32x16& cur = s[kb & 1];
         f32x16& nxt = s[(kb + 1) & 1];
-        // rare path: raise the reference max and rescale what has been accumulated
-        const bool raise = mx_cur > m_run + kRescaleTau;
-        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+        // raise the reference max of the lanes in `raise` to at least m_block and rescale what has been accumulated
+        auto raise_reference = [&](bool raise, float m_block) {
             // the accumulating MFMAs of the previous step must have left the pipeline
             asm volatile("s_nop 15\n\ts_nop 15" : "+v"(tok));
-            const float m_new = raise ? mx_cur : m_run;
+            const float m_new = raise ? fmaxf(m_run, m_block) : m_run;
             const float m_use_new = (m_new == -INFINITY) ? 0.f : m_new;
             const float alpha = fast_exp2(m_use - m_use_new);
             m_run = m_new;
@@ -196,19 +198,49 @@ __device__ __forceinline__ void fwd_q_tile_regs(const FwdParams& p, char* smem, 
             l_run *= alpha;
             static_for<DB>([&](auto db) { agpr_scale_block<O_BASE + 16 * db>(alpha, tok); });
             asm volatile("s_nop 3" : "+v"(tok));
+        };
+        if constexpr (!kGuard) {
+            // rare path: the block max computed in the previous step exceeds the reference by more than tau
+            const bool raise = mx_cur > m_run + kRescaleTau;
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) raise_reference(raise, mx_cur);
         }
         const bool have_next = kb + 1 < KB;
         // scores of the next step fly while this step's softmax runs
         if (have_next) scores(nxt, stage, kb + 1);
         float psum = 0.f;
+        i32x4 pb[2];
+        // P against the reference the row has, packed at once; the raw scores stay in `cur`
+        auto softmax_block = [&]() {
+            psum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            float pv = fast_exp2(__builtin_fmaf(cur[r], scale, -m_use));
-            cur[r] = pv;
-            psum += pv;
+            for (int s2 = 0; s2 < 2; s2++) {
+                f32x8 ps;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    ps[e] = fast_exp2(__builtin_fmaf(cur[8 * s2 + e], scale, -m_use));
+                    psum += ps[e];
+                }
+                pb[s2] = Elem<E>::pack8(ps);
+            }
+        };
+        softmax_block();
+        if constexpr (kGuard) {
+            // Guarded softmax, as in fwd_kernel: a row keeps the max of its first visible block as reference
+            // while the block sums stay below guard_above; a row without reference has guard_above = -1.
+            const unsigned long long fired = __builtin_amdgcn_ballot_w64(psum > guard_above);
+            if (fired != 0) {
+                // the two lanes of a row (l and l ^ 32) hold half of its keys each and share its reference
+                const bool fire = (((fired | (fired >> 32) | (fired << 32)) >> lane) & 1) != 0;
+                float mx = cur[0];
+#pragma unroll
+                for (int r = 1; r < 16; r++) mx = fmaxf(mx, cur[r]);
+                raise_reference(fire, max_across_halves(mx) * scale);
+                guard_above = (m_run == -INFINITY) ? -1.f : kGuardLimit;
+                softmax_block();
+            }
         }
         l_run += psum;
-        accumulate(cur, stage, kb);
+        accumulate(pb, stage, kb);
         if (have_next) mx_cur = prepare(nxt, full, k0 + 32 * (kb + 1));
     };
 

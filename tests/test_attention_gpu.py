@@ -143,13 +143,14 @@ def test_lse_and_fully_masked_rows():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("dtype,growth", [(torch.float16, 60.0), (torch.bfloat16, 400.0), (torch.float32, 60.0)], ids=str)
-def test_reference_max_is_raised_along_the_keys(dtype, growth):
+def test_reference_max_is_raised_along_the_keys(dtype, growth, D):
     """Scores that grow by `growth` (log2 units) along the key axis: the forward's reference max has to be
     raised many times per row (16-bit inputs: whenever a block's sum of P leaves the guarded range), in rows
     whose two half-wave lanes see different sums.  Same bar as the other forward tests."""
     torch.manual_seed(7)
-    B, H, T, D = 1, 2, 1024, 64
+    B, H, T = 1, 2, 1024
     q = torch.randn(B, H, T, D, device=DEV) * 0.5
     k = torch.randn(B, H, T, D, device=DEV) * 0.5
     v = torch.randn(B, H, T, D, device=DEV)
@@ -164,6 +165,10 @@ def test_reference_max_is_raised_along_the_keys(dtype, growth):
         ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), None)
         out, lse = ca.chill_attention(q, k, v, mask=mask, return_lse=True)
         atol, rtol = OUT_TOL[dtype]
+        if dtype == torch.float32:
+            # raw scores reach several hundred here: their fp32 rounding alone moves P by ~3e-5 relative, whatever
+            # the order of the sums, so the fp32 bar of the other tests (2e-6 / 1e-4) is out of reach for both sides
+            atol, rtol = 1e-5, 1e-3
         assert torch.isfinite(out).all() and torch.isfinite(lse).all()
         torch.testing.assert_close(out * res_mask, ref.to(dtype), atol=atol, rtol=rtol)
 
