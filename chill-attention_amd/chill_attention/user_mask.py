@@ -71,7 +71,8 @@ def functor_source(cls) -> str:
 def _kernel_sources_digest() -> bytes:
     h = hashlib.sha1()
     for name in sorted(os.listdir(CSRC_DIR)):
-        if name.endswith((".h", ".hip", ".cpp")) or name == "Makefile":
+        # (the generated .inc files follow from the .py generators)
+        if name.endswith((".h", ".hip", ".cpp", ".py")) or name == "Makefile":
             with open(os.path.join(CSRC_DIR, name), "rb") as f:
                 h.update(name.encode() + b"\0" + f.read())
     return h.digest()

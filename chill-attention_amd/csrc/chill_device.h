@@ -66,6 +66,11 @@ struct Elem<bf16_t> {
     __device__ __forceinline__ static i32x2 pack4(f32x4 v) {
         return __builtin_bit_cast(i32x2, __builtin_convertvector(v, bf16x4));
     }
+    __device__ __forceinline__ static int pack2(float lo, float hi) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(int, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
+    }
     __device__ __forceinline__ static float to_float(type x) { return (float)x; }
 };
 
@@ -84,6 +89,11 @@ struct Elem<f16_t> {
     }
     __device__ __forceinline__ static i32x2 pack4(f32x4 v) {
         return __builtin_bit_cast(i32x2, __builtin_convertvector(v, f16x4));
+    }
+    __device__ __forceinline__ static int pack2(float lo, float hi) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_bit_cast(int, __builtin_convertvector(f32x2{lo, hi}, f16x2));
     }
     __device__ __forceinline__ static float to_float(type x) { return (float)x; }
 };

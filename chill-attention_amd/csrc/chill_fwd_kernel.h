@@ -404,14 +404,51 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
 
 }  // namespace chill
 #include "chill_fwd_regs.h"
+#include "chill_fwd_fast.h"
 namespace chill {
+
+// Shapes served by fwd_q_tile_fast (16-bit inputs, head dim 64 or 128, 64-key tiles with one resident
+// ahead); fwd_q_tile stays behind it for the q-tiles whose sums leave the range it is exact in.
+template <typename E, int D, int TK, int NS>
+constexpr bool fwd_is_fast() {
+    return CHILL_FWD_FAST && Elem<E>::k16 && (D == 64 || D == 128) && TK == 64 && NS >= 3;
+}
+template <typename E, int D, int TK, int NS>
+constexpr int fwd_lds_bytes() {
+    return NS * FwdLds<E, D, TK>::STAGE_BYTES + (fwd_is_fast<E, D, TK, NS>() ? kFwdFastFlagBytes : 0);
+}
+
+// true if `mine` is true for any wave of the workgroup; flags = one int per wave in LDS
+template <int NW>
+__device__ __forceinline__ bool workgroup_any(bool mine, char* flags) {
+    volatile int* f = reinterpret_cast<volatile int*>(flags);
+    if ((threadIdx.x & 63) == 0) f[threadIdx.x >> 6] = mine ? 1 : 0;
+    __syncthreads();
+    int any = 0;
+#pragma unroll
+    for (int w = 0; w < NW; w++) any |= f[w];
+    __syncthreads();  // the flags and the ring are reused
+    return any != 0;
+}
+
+template <typename E, int D, int MASK, int NW, int TK, int NS>
+__device__ __forceinline__ void fwd_one_q_tile(const FwdParams& p, char* smem, int b, int hd, int qt,
+                                               int wave_has_full_blocks) {
+    if constexpr (fwd_is_fast<E, D, TK, NS>()) {
+        const bool again = fwd_q_tile_fast<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt);
+        if (workgroup_any<NW>(again, smem + NS * FwdLds<E, D, TK>::STAGE_BYTES))
+            fwd_q_tile<E, D, MASK, NW, TK, 3>(p, smem, b, hd, qt, wave_has_full_blocks);
+    } else {
+        fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt, wave_has_full_blocks);
+    }
+}
 
 // Workgroups of four waves whose LDS ring leaves room for a second workgroup on the CU are compiled
 // for 256 registers per wave, so that two of them share a CU: one computes while the other loads its
 // first tiles or stores its result.
 template <typename E, int D, int NW, int TK, int NS>
 constexpr int fwd_waves_per_simd() {
-    return (NW == 4 && Elem<E>::k16 && 2 * NS * FwdLds<E, D, TK>::STAGE_BYTES <= 160 * 1024) ? 2 : 1;
+    return (NW == 4 && Elem<E>::k16 && 2 * fwd_lds_bytes<E, D, TK, NS>() <= 160 * 1024) ? 2 : 1;
 }
 
 // One workgroup per (batch, head, PAIR of q-tiles): tile j from the end, then tile j from the
@@ -432,10 +469,10 @@ void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
     const int b = bh / p.H;
     const int hd = bh % p.H;
     const int qt_hi = n_q_tiles - 1 - j;
-    fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, wave_has_full_blocks);
+    fwd_one_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, wave_has_full_blocks);
     if (paired && j != qt_hi) {
         __syncthreads();  // the LDS ring is reused
-        fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
+        fwd_one_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
     }
 }
 
@@ -453,6 +490,7 @@ int launch_fwd_shape(const FwdParams& p, hipStream_t stream) {
     static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
     constexpr int NS = fwd_stages(MASK_ID, D, Elem<E>::kDType, kRowFor);
     static_assert(cfg.lds_bytes == NS * FwdLds<E, D, cfg.streamed>::STAGE_BYTES, "table and kernel disagree on LDS");
+    constexpr int kLdsBytes = fwd_uses_regs(D, Elem<E>::kDType) ? cfg.lds_bytes : fwd_lds_bytes<E, D, cfg.streamed, NS>();
     const int n_q_tiles = cdiv(p.T, cfg.rows);
     // pairing q-tiles balances long causal runs; with few workgroups it only halves the number of
     // CUs that get work
@@ -467,12 +505,12 @@ int launch_fwd_shape(const FwdParams& p, hipStream_t stream) {
     else
         kern = fwd_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
     const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
-    if (cfg.lds_bytes > 48 * 1024) {
+    if (kLdsBytes > 48 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                cfg.lds_bytes) != hipSuccess)
+                                kLdsBytes) != hipSuccess)
             return CHILL_ERR_HIP;
     }
-    hipLaunchKernelGGL(kern, grid, block, cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0, paired ? 1 : 0);
+    hipLaunchKernelGGL(kern, grid, block, kLdsBytes, stream, p, n_q_tiles, total, hfb ? 1 : 0, paired ? 1 : 0);
     return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
 }
 

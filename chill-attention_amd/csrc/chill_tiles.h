@@ -37,6 +37,13 @@
 #define CHILL_TUNE_DKDV_R64 0
 #endif
 
+// 1: the 8-wave forward of 16-bit inputs at head dim 128 streams 64-key tiles through four stages,
+// the shape fwd_q_tile_fast and its generated loop are written for; 0: the shape before it (128-key
+// tiles, two stages, fwd_q_tile).
+#ifndef CHILL_FWD_FAST
+#define CHILL_FWD_FAST 1
+#endif
+
 namespace chill {
 
 constexpr int elem_bytes(int dtype) { return dtype == CHILL_F32 ? 4 : 2; }
@@ -89,7 +96,7 @@ constexpr int fwd_streamed(int mask_id, int D, int dtype, int T) {
     if (dtype == CHILL_F32) return 32;
     if (D > 128) return 64;
     if (CHILL_TUNE_FWD_STREAMED) return CHILL_TUNE_FWD_STREAMED;
-    return fwd_waves(mask_id, D, dtype, T) == 8 ? 128 : 64;
+    return (fwd_waves(mask_id, D, dtype, T) == 8 && !CHILL_FWD_FAST) ? 128 : 64;
 }
 // LDS stages of the forward K/V ring: two for the 4-wave shape of 16-bit inputs (so that two
 // workgroups fit a CU); otherwise three (one tile resident ahead, one in flight) when they fit in
@@ -99,6 +106,7 @@ constexpr int fwd_stages(int mask_id, int D, int dtype, int T) {
     if (dtype != CHILL_F32 && D <= 128) {
         if (CHILL_TUNE_FWD_STAGES) return CHILL_TUNE_FWD_STAGES;
         if (fwd_waves(mask_id, D, dtype, T) == 4) return 2;
+        if (CHILL_FWD_FAST) return 4;
     }
     return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
 }
