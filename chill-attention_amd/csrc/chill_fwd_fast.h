@@ -62,10 +62,29 @@ __device__ __forceinline__ i32x4 scale_chunk(i32x4 c, float f) {
     return Elem<E>::pack8(x);
 }
 
-// Returns true (wave-uniform) when a row of this wave left the range the reference-free softmax is
-// exact in; the outputs of the q-tile are then to be computed again by fwd_q_tile.
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ unsigned uniform(unsigned x) { return (unsigned)__builtin_amdgcn_readfirstlane((int)x); }
+
+// true if `mine` is true for any wave of the workgroup; flags = one int per wave in LDS
+template <int NW>
+__device__ __forceinline__ bool workgroup_any(bool mine, char* flags) {
+    volatile int* f = reinterpret_cast<volatile int*>(flags);
+    if ((threadIdx.x & 63) == 0) f[threadIdx.x >> 6] = mine ? 1 : 0;
+    __syncthreads();
+    int any = 0;
+#pragma unroll
+    for (int w = 0; w < NW; w++) any |= f[w];
+    __syncthreads();  // the flags are reused
+    return __builtin_amdgcn_readfirstlane(any) != 0;  // (the same in every lane: say so to the compiler)
+}
+
+// The q-tiles qt_a and then qt_b (-1: none) of one head, start to finish.  While the rows of one q-tile
+// are normalised and stored, the first K/V tiles and the Q rows of the next one are already on their
+// way.  A q-tile in which a row left the range the reference-free softmax is exact in is computed
+// again by fwd_q_tile.
 template <typename E, int D, int MASK, int NW, int TK, int NS>
-__device__ __forceinline__ bool fwd_q_tile_fast(const FwdParams& p, char* smem, int b, int hd, int qt) {
+__device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem, int b, int hd, int qt_a, int qt_b,
+                                                 int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
     using M = Mask<MASK>;
     typedef FwdLds<E, D, TK> Lds;
@@ -91,73 +110,31 @@ __device__ __forceinline__ bool fwd_q_tile_fast(const FwdParams& p, char* smem, 
     int seq_len = p.T;
     if (p.lens != nullptr) seq_len = imin(p.lens[(int64_t)b * p.lens_stride], p.T);
 
-    const int qb = qt * TQ;
     ET* obase = reinterpret_cast<ET*>(p.o) + b * p.so.b + hd * p.so.h;
     float* lse_base = p.lse ? p.lse + b * p.lse_b + hd * p.lse_h : nullptr;
-
-    if (qb >= seq_len) {
-        // nothing attends here: the output rows are defined to be zero (chill.py:96, chill_fwd.py:70-71)
-        int nrows = imin(TQ, p.T - qb);
-        zero_rows<E, D, NT>(obase, p.so.t, qb, nrows, tid);
-        if (lse_base)
-            for (int i = tid; i < nrows; i += NT) lse_base[qb + i] = 0.f;
-        return false;
-    }
-
     const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hd * p.sq.h;
     const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
     const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
 
-    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
-    const int n_tiles = wg.end - wg.start;
     AsyncPaddedLoader<E, D, rowwise_pad<E, D>(), TK, NT> load_k;
     AsyncPaddedLoader<E, D, transposed_pad<E, D>(), TK, NT> load_v;
     load_k.init(p.sk.t, wave, lane);
     load_v.init(p.sv.t, wave, lane);
     // every wave issues at least this many loads per tile
     constexpr int kLoadsPerTile = decltype(load_k)::SLABS / NW + decltype(load_v)::SLABS / NW;
-    auto issue_tile = [&](int i, int st_index) {
-        int k0 = (wg.start + i) * TK;
+    // tile `tile` (absolute index along the keys) into LDS stage st_index
+    auto issue_tile = [&](int tile, int st_index) {
+        int k0 = tile * TK;
         char* st = smem + st_index * Lds::STAGE_BYTES;
         load_k.issue(kptr + (int64_t)k0 * p.sk.t, p.sk.t, p.T - k0, st, wave, lane);
         load_v.issue(vptr + (int64_t)k0 * p.sv.t, p.sv.t, p.T - k0, st + Lds::K_BYTES, wave, lane);
     };
-    // stores of an earlier q-tile must not be counted among the tile loads
-    wait_async_tiles();
-#pragma unroll
-    for (int i = 0; i <= 1 + FL; i++)
-        if (i < n_tiles) issue_tile(i, i);
-
-    const int qw = qb + 32 * wave;
-    Resident<E, D> qf;
-    load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
-
-    // this wave's 32-key blocks, as steps counted from the first block of the workgroup's first tile
-    int g0 = 0, g1 = 0, f0 = 0, f1 = 0;
-    if (qw < seq_len) {
-        const TileRange wr = tile_range<MASK, true>(qw, 32, 32, seq_len, M::has_full_blocks(32, 32, p.T, p.margs), p.margs);
-        const int base = wg.start * KB;
-        g0 = imax(wr.start - base, 0);
-        g1 = imin(wr.end - base, n_tiles * KB);
-        f0 = wr.full_start - base;
-        f1 = wr.full_end - base;
-    }
 
     // per-lane LDS offsets inside a stage; everything else is an immediate
     const int k_lane = n * KT::PITCH + h * 16;
     const int r16 = lane & 15, colgrp = (lane >> 4) & 1;
     const int v_lane = Lds::K_BYTES + (4 * h + (r16 >> 2)) * VT::PITCH + (16 * colgrp + 4 * (r16 & 3)) * 2;
-
-    f32x16 o[DB];
-#pragma unroll
-    for (int i = 0; i < DB; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o[i][r] = 0.f;
-    float l_run = 0.f;   // this lane's share of the row sum
-    float m0 = 0.f;      // the row's reference (log2 domain, scale included)
-    bool over = false;   // fp16: a block sum went above the limit
-    const int q_pos = qw + n;
-    const Range vis = visible_range<MASK, true>(q_pos, seq_len, p.margs);  // the keys this lane's row sees
+    const lds_char* lds0 = (const lds_char*)smem;
 
     struct KOperands {
         i32x4 c[NJ];
@@ -182,181 +159,299 @@ __device__ __forceinline__ bool fwd_q_tile_fast(const FwdParams& p, char* smem, 
                 vo.hi[s2][db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4*)(a0 + 8 * VT::PITCH));
             }
     };
-    auto mask_block = [&](f32x16& sc, int key0) {
-        if constexpr (M::kRowIsRange) {
-            fill_outside_range(sc, vis.lo, vis.hi, key0 + 4 * h, -INFINITY);
-        } else {
+
+    // What is on its way for the next q-tile: the tiles of its hull wg_pre (the first NS - 1 of them,
+    // tile i in stage i) and its Q rows in qf.
+    Resident<E, D> qf;
+    TileRange wg_pre = {0, 0, 0, 0};
+    auto prefetch = [&](int qt) {
+        const int qb = qt * TQ;
+        wg_pre = TileRange{0, 0, 0, 0};
+        if (qb >= seq_len) return;
+        wg_pre = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
-                bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
-                sc[r] = ok ? sc[r] : -INFINITY;
-            }
-        }
+        for (int i = 0; i <= 1 + FL; i++)
+            if (wg_pre.start + i < wg_pre.end) issue_tile(wg_pre.start + i, i);
+        const int qw = qb + 32 * wave;
+        load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
     };
+    prefetch(qt_a);
+#ifdef CHILL_FWD_TIMING
+    // instrumented build: wave 0 leaves 100 MHz timestamps of its phases in the LSE rows of its q-tile
+    unsigned stamps[8];
+#define CHILL_STAMP(i) stamps[i] = (unsigned)__builtin_amdgcn_s_memrealtime()
+#else
+#define CHILL_STAMP(i)
+#endif
 
-    // Q: wait for it, fold the scale in (a negative scale needs nothing special here)
-#pragma unroll
-    for (int j = 0; j < NJ; j++) {
-        qf.c[j] = scale_chunk<E>(qf.c[j], p.scale_log2);
-        asm volatile("" : "+v"(qf.c[j]));
-    }
-
-    f32x16 mneg;  // the accumulator block the score chains start from: -m0 everywhere
-#pragma unroll
-    for (int r = 0; r < 16; r++) mneg[r] = 0.f;
-    const lds_char* lds0 = (const lds_char*)smem;
-
-    bool have_ref = false;  // wave-uniform: the rows have their reference
-    // One step outside the generated loop, from the scores to O: block g of the wave (the first one
-    // also settles the row's reference).  Not pipelined: the first and the last few blocks of a wave,
-    // and every block that needs the mask, come here.
-    auto plain_step = [&](const lds_char* stage, int kb, int g) {
-        KOperands ka;
-        k_read(ka, stage, kb);
-        f32x16 sc = Elem<E>::mma(ka.c[0], qf.c[0], mneg);
-#pragma unroll
-        for (int j = 1; j < NJ; j++) sc = Elem<E>::mma(ka.c[j], qf.c[j], sc);
-        if (g < f0 || g >= f1) mask_block(sc, (wg.start * KB + g) * 32);
-        if (!have_ref) {
-            have_ref = true;
-            float mx = sc[0];
-#pragma unroll
-            for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
-            mx = max_across_halves(mx);
-            m0 = (mx == -INFINITY) ? 0.f : mx;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                mneg[r] = -m0;
-                sc[r] -= m0;
-            }
-            asm volatile("" : "+v"(mneg));  // sixteen registers, not one value the compiler may splat again
+#pragma nounroll
+    for (int item = 0; item < 2; item++) {
+        const int qt = item == 0 ? qt_a : qt_b;
+        const int qt_next = item == 0 ? qt_b : -1;
+        if (qt < 0) break;
+        const int qb = qt * TQ;
+        if (qb >= seq_len) {
+            // nothing attends here: the output rows are defined to be zero (chill.py:96, chill_fwd.py:70-71)
+            int nrows = imin(TQ, p.T - qb);
+            zero_rows<E, D, NT>(obase, p.so.t, qb, nrows, tid);
+            if (lse_base)
+                for (int i = tid; i < nrows; i += NT) lse_base[qb + i] = 0.f;
+#ifndef CHILL_FWD_NO_PREFETCH
+            if (qt_next >= 0) prefetch(qt_next);
+#endif
+            continue;
         }
-        VOperands vo;
-        v_read(vo, stage, kb);
-        float psum = 0.f;
-        i32x4 pb[2];
-#pragma unroll
-        for (int s2 = 0; s2 < 2; s2++) {
-            f32x8 ps;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                ps[e] = fast_exp2(sc[8 * s2 + e]);
-                psum += ps[e];
-            }
-            pb[s2] = Elem<E>::pack8(ps);
-        }
-        if (Lim::kBlockLimit) over |= psum > Lim::kBlockHi;
-        l_run += psum;
-#pragma unroll
-        for (int s2 = 0; s2 < 2; s2++)
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                i16x8 av = __builtin_shufflevector(vo.lo[s2][db], vo.hi[s2][db], 0, 1, 2, 3, 4, 5, 6, 7);
-                o[db] = Elem<E>::mma(__builtin_bit_cast(i32x4, av), pb[s2], o[db]);
-            }
-    };
+        CHILL_STAMP(0);
+#ifdef CHILL_FWD_NO_PREFETCH
+        if (item > 0) prefetch(qt);
+#endif
+        const TileRange wg = {uniform(wg_pre.start), uniform(wg_pre.end), 0, 0};
+        const int n_tiles = wg.end - wg.start;
+        const int qw = qb + 32 * wave;
 
-    // Tiles [i_lo, i_hi) go to the generated loop: both blocks inside the wave's range and
-    // predicate-free.
-    int i_lo = (imax(g0, f0) + KB - 1) / KB;
-    int i_hi = imin(imin(g1, f1) / KB, n_tiles);
-    // a tile that ends past T is zero-filled by its loader, which the generated loop does not do
-    if (p.T % TK != 0) i_hi = imin(i_hi, p.T / TK - wg.start - (NS - 1));
-    if (!fwd_has_generated_loop<E, D, NW, NS>() || g1 <= g0 || i_hi < i_lo) i_lo = i_hi = 0;
-
-    int st_cur = NS - 1;  // LDS stage of tile i (advanced at the top of the loop)
-    // tiles <= i + 1 have landed for every wave, and everyone is done with tile i - 1
-    auto ring_top = [&](int i) {
-        if (FL > 0 && i + 1 + FL < n_tiles)
-            wait_async_tiles_except<FL * kLoadsPerTile>();
-        else
-            wait_async_tiles();
-        __syncthreads();
-        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
-        if (i + NS - 1 < n_tiles) issue_tile(i + NS - 1, st_cur == 0 ? NS - 1 : st_cur - 1);
-    };
-    auto plain_tile = [&](int i) {
-        ring_top(i);
-        const lds_char* stage = lds0 + st_cur * Lds::STAGE_BYTES;
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++) {
-            const int g = i * KB + kb;
-            if (g >= g0 && g < g1) plain_step(stage, kb, g);
+        // this wave's 32-key blocks, as steps counted from the first block of the workgroup's first tile
+        int g0 = 0, g1 = 0, f0 = 0, f1 = 0;
+        if (qw < seq_len) {
+            const TileRange wr =
+                tile_range<MASK, true>(qw, 32, 32, seq_len, M::has_full_blocks(32, 32, p.T, p.margs), p.margs);
+            const int base = wg.start * KB;
+            g0 = imax(wr.start - base, 0);
+            g1 = imin(wr.end - base, n_tiles * KB);
+            f0 = wr.full_start - base;
+            f1 = wr.full_end - base;
         }
-    };
-    int i = 0;
-    for (; i < i_lo || (i_lo == i_hi && i < n_tiles); i++) plain_tile(i);
-    if constexpr (fwd_has_generated_loop<E, D, NW, NS>()) {
-        if (i_hi > i_lo) {
-            ring_top(i_lo);
+
+        f32x16 o[DB];
+#pragma unroll
+        for (int i = 0; i < DB; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[i][r] = 0.f;
+        float l_run = 0.f;   // this lane's share of the row sum
+        float m0 = 0.f;      // the row's reference (log2 domain, scale included)
+        bool over = false;   // fp16: a block sum went above the limit
+        const int q_pos = qw + n;
+        const Range vis = visible_range<MASK, true>(q_pos, seq_len, p.margs);  // the keys this lane's row sees
+
+        auto mask_block = [&](f32x16& sc, int key0) {
+            if constexpr (M::kRowIsRange) {
+                fill_outside_range(sc, vis.lo, vis.hi, key0 + 4 * h, -INFINITY);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+                    bool ok = (key < seq_len) && M::pred(q_pos, key, seq_len, p.margs);
+                    sc[r] = ok ? sc[r] : -INFINITY;
+                }
+            }
+        };
+
+        // Q: wait for it, fold the scale in (a negative scale needs nothing special here)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            qf.c[j] = scale_chunk<E>(qf.c[j], p.scale_log2);
+            asm volatile("" : "+v"(qf.c[j]));
+        }
+
+        f32x16 mneg;  // the accumulator block the score chains start from: -m0 everywhere
+#pragma unroll
+        for (int r = 0; r < 16; r++) mneg[r] = 0.f;
+        CHILL_STAMP(1);
+
+        bool have_ref = false;  // wave-uniform: the rows have their reference
+        // One step outside the generated loop, from the scores to O: block g of the wave (the first one
+        // also settles the row's reference).  Not pipelined: the first and the last few blocks of a wave,
+        // and every block that needs the mask, come here.
+        auto plain_step = [&](const lds_char* stage, int kb, int g) {
+            KOperands ka;
+            k_read(ka, stage, kb);
+            f32x16 sc = Elem<E>::mma(ka.c[0], qf.c[0], mneg);
+#pragma unroll
+            for (int j = 1; j < NJ; j++) sc = Elem<E>::mma(ka.c[j], qf.c[j], sc);
+            if (g < f0 || g >= f1) mask_block(sc, (wg.start * KB + g) * 32);
             if (!have_ref) {
-                // the wave starts here: the reference comes from its first block, whose scores the
-                // loop computes again
                 have_ref = true;
-                KOperands ka;
-                k_read(ka, lds0 + st_cur * Lds::STAGE_BYTES, 0);
-                f32x16 sc = Elem<E>::mma(ka.c[0], qf.c[0], mneg);
-#pragma unroll
-                for (int j = 1; j < NJ; j++) sc = Elem<E>::mma(ka.c[j], qf.c[j], sc);
                 float mx = sc[0];
 #pragma unroll
                 for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
-                m0 = max_across_halves(mx);
+                mx = max_across_halves(mx);
+                m0 = (mx == -INFINITY) ? 0.f : mx;
 #pragma unroll
-                for (int r = 0; r < 16; r++) mneg[r] = -m0;
-                asm volatile("" : "+v"(mneg));
-            }
-            int cnt = i_hi - i_lo;
-            int rem = n_tiles - i_lo - 3;            // tiles behind the one the next barrier certifies
-            const unsigned lds_base = lds_address(smem);
-            unsigned cur = lds_base + st_cur * Lds::STAGE_BYTES;   // stage of tile i_lo
-            const int64_t t_issue = (int64_t)(wg.start + i_lo + NS) * TK;  // first key of the next tile to load
-            const ET* kb = kptr + t_issue * p.sk.t;
-            const ET* vb = vptr + t_issue * p.sv.t;
-            const unsigned kstep = (unsigned)(TK * p.sk.t * Elem<E>::kBytes), vstep = (unsigned)(TK * p.sv.t * Elem<E>::kBytes);
-            const unsigned w1024 = wave * 1024;
-            i32x16 q0, q1;
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    q0[4 * j + e] = qf.c[j][e];
-                    q1[4 * j + e] = qf.c[4 + j][e];
+                for (int r = 0; r < 16; r++) {
+                    mneg[r] = -m0;
+                    sc[r] -= m0;
                 }
-            if constexpr (std::is_same<E, bf16_t>::value) {
-                CHILL_FWD_LOOP_BF16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, q0, q1, mneg, k_lane, v_lane,
-                                            load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0], load_v.goff[1],
-                                            load_v.goff[2], lds_base, kstep, vstep, w1024, wave);
-            } else {
-                unsigned long long over_mask = 0;
-                const float block_hi = Lim::kBlockHi;
-                CHILL_FWD_LOOP_F16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, over_mask, q0, q1, mneg, k_lane,
-                                           v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
-                                           load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
-                over |= ((over_mask >> lane) & 1) != 0;
+                asm volatile("" : "+v"(mneg));  // sixteen registers, not one value the compiler may splat again
             }
-            st_cur = (st_cur + (i_hi - i_lo - 1)) % NS;
-            i = i_hi;
+            VOperands vo;
+            v_read(vo, stage, kb);
+            float psum = 0.f;
+            i32x4 pb[2];
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                f32x8 ps;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    ps[e] = fast_exp2(sc[8 * s2 + e]);
+                    psum += ps[e];
+                }
+                pb[s2] = Elem<E>::pack8(ps);
+            }
+            if (Lim::kBlockLimit) over |= psum > Lim::kBlockHi;
+            l_run += psum;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    i16x8 av = __builtin_shufflevector(vo.lo[s2][db], vo.hi[s2][db], 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = Elem<E>::mma(__builtin_bit_cast(i32x4, av), pb[s2], o[db]);
+                }
+        };
+
+        // Tiles [i_lo, i_hi) go to the generated loop: both blocks inside the wave's range and
+        // predicate-free.
+        int i_lo = (imax(g0, f0) + KB - 1) / KB;
+        int i_hi = imin(imin(g1, f1) / KB, n_tiles);
+        // a tile that ends past T is zero-filled by its loader, which the generated loop does not do
+        if (p.T % TK != 0) i_hi = imin(i_hi, p.T / TK - wg.start - (NS - 1));
+        if (!fwd_has_generated_loop<E, D, NW, NS>() || g1 <= g0 || i_hi < i_lo) i_lo = i_hi = 0;
+
+        int st_cur = NS - 1;  // LDS stage of tile i (advanced at the top of the loop)
+        // Tiles <= i + 1 have landed for every wave, and everyone is done with tile i - 1.  The first wait
+        // of a q-tile is for everything: the stores of the q-tile before are among what is outstanding,
+        // and they do not complete in order with the loads.
+        auto ring_top = [&](int i, bool issue) {
+            if (FL > 0 && i > 0 && i + 1 + FL < n_tiles)
+                wait_async_tiles_except<FL * kLoadsPerTile>();
+            else
+                wait_async_tiles();
+            __syncthreads();
+            st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
+            if (issue && i + NS - 1 < n_tiles) issue_tile(wg.start + i + NS - 1, st_cur == 0 ? NS - 1 : st_cur - 1);
+        };
+        auto plain_tile = [&](int i) {
+            ring_top(i, true);
+            const lds_char* stage = lds0 + st_cur * Lds::STAGE_BYTES;
+#pragma unroll
+            for (int kb = 0; kb < KB; kb++) {
+                const int g = i * KB + kb;
+                if (g >= g0 && g < g1) plain_step(stage, kb, g);
+            }
+        };
+        int i = 0;
+        for (; i < i_lo || (i_lo == i_hi && i < n_tiles); i++) plain_tile(i);
+        CHILL_STAMP(2);
+        if constexpr (fwd_has_generated_loop<E, D, NW, NS>()) {
+            if (i_hi > i_lo) {
+                ring_top(i_lo, false);  // the generated loop issues the tile that is due here
+                CHILL_STAMP(3);
+#ifdef CHILL_FWD_TIMING
+                const unsigned clk0 = (unsigned)__builtin_amdgcn_s_memtime();
+#endif
+                if (!have_ref) {
+                    // the wave starts here: the reference comes from its first block, whose scores the
+                    // loop computes again
+                    have_ref = true;
+                    KOperands ka;
+                    k_read(ka, lds0 + st_cur * Lds::STAGE_BYTES, 0);
+                    f32x16 sc = Elem<E>::mma(ka.c[0], qf.c[0], mneg);
+#pragma unroll
+                    for (int j = 1; j < NJ; j++) sc = Elem<E>::mma(ka.c[j], qf.c[j], sc);
+                    float mx = sc[0];
+#pragma unroll
+                    for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
+                    m0 = max_across_halves(mx);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) mneg[r] = -m0;
+                    asm volatile("" : "+v"(mneg));
+                }
+                // (all of these are the same in every lane; uniform() says so where the compiler has lost track)
+                int cnt = uniform(i_hi - i_lo);
+                int rem = uniform(n_tiles - i_lo - 2);   // tiles behind the one the last barrier certified
+                const unsigned lds_base = lds_address(smem);
+                unsigned cur = uniform(lds_base + st_cur * Lds::STAGE_BYTES);   // stage of tile i_lo
+                const int t_issue = uniform((wg.start + i_lo + NS - 1) * TK);  // first key of the next tile to load
+                const ET* kb = kptr + (int64_t)t_issue * p.sk.t;
+                const ET* vb = vptr + (int64_t)t_issue * p.sv.t;
+                const unsigned kstep = (unsigned)(TK * p.sk.t * Elem<E>::kBytes), vstep = (unsigned)(TK * p.sv.t * Elem<E>::kBytes);
+                const unsigned w1024 = wave * 1024;
+                i32x16 q0, q1;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        q0[4 * j + e] = qf.c[j][e];
+                        q1[4 * j + e] = qf.c[4 + j][e];
+                    }
+                if constexpr (std::is_same<E, bf16_t>::value) {
+                    CHILL_FWD_LOOP_BF16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, q0, q1, mneg, k_lane,
+                                                v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
+                                                load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave);
+                } else {
+                    unsigned long long over_mask = 0;
+                    const float block_hi = Lim::kBlockHi;
+                    CHILL_FWD_LOOP_F16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, over_mask, q0, q1, mneg,
+                                               k_lane, v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
+                                               load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
+                    over |= ((over_mask >> lane) & 1) != 0;
+                }
+                CHILL_STAMP(4);
+#ifdef CHILL_FWD_TIMING
+                stamps[1] = (unsigned)__builtin_amdgcn_s_memtime() - clk0;  // shader clocks spent in the loop
+#endif
+                st_cur = (st_cur + (i_hi - i_lo - 1)) % NS;
+                i = i_hi;
+            }
+        }
+        for (; i < n_tiles; i++) plain_tile(i);
+        CHILL_STAMP(5);
+
+        // the ring is free once every wave is here: start on the next q-tile before this one is stored
+#ifndef CHILL_FWD_NO_PREFETCH
+        if (qt_next >= 0) {
+            __syncthreads();
+            prefetch(qt_next);
+        }
+#endif
+        CHILL_STAMP(6);
+
+        // epilogue: O = acc / l, LSE2 = m0 + log2(l) (chill_fwd.py:288-289, 327-328)
+        const float l_tot = sum_across_halves(l_run);
+        const float l_safe = (l_tot == 0.f) ? 1.f : l_tot;
+        const float inv = 1.f / l_safe;
+        const bool valid = q_pos < seq_len;
+        const bool in_t = q_pos < p.T;
+        if (in_t) {
+            ET* orow = obase + (int64_t)q_pos * p.so.t;
+            store_row_transposed<E, D>(orow, o, inv, valid, h);
+            if (lse_base != nullptr && h == 0)
+                lse_base[q_pos] = valid ? (l_tot == 0.f ? -INFINITY : m0 + __log2f(l_tot)) : 0.f;
+        }
+        // a row that sees keys must end with a sum inside the range (a NaN fails the comparison too)
+        const bool bad = (vis.lo <= vis.hi) && (over || !(l_tot >= Lim::kLo && l_tot <= Lim::kHi));
+        const bool again = __builtin_amdgcn_ballot_w64(bad) != 0;
+#ifdef CHILL_FWD_TIMING
+        CHILL_STAMP(7);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (wave == 0 && lane == 0 && lse_base != nullptr && qb + 9 <= p.T) {
+            unsigned end = (unsigned)__builtin_amdgcn_s_memrealtime();
+#pragma unroll
+            for (int t = 0; t < 8; t++) lse_base[qb + t] = __builtin_bit_cast(float, stamps[t]);
+            lse_base[qb + 8] = __builtin_bit_cast(float, end);
+        }
+#endif
+        if (workgroup_any<NW>(again, smem + NS * Lds::STAGE_BYTES)) {
+            // rare: give the ring to the kernel whose softmax follows the running max, then start over on
+            // the next q-tile
+            wait_async_tiles();
+            __syncthreads();
+            fwd_q_tile<E, D, MASK, NW, TK, 3>(p, smem, b, hd, qt, wave_has_full_blocks);
+            __syncthreads();
+#ifndef CHILL_FWD_NO_PREFETCH
+            if (qt_next >= 0) prefetch(qt_next);
+#endif
         }
     }
-    for (; i < n_tiles; i++) plain_tile(i);
-
-    // epilogue: O = acc / l, LSE2 = m0 + log2(l) (chill_fwd.py:288-289, 327-328)
-    const float l_tot = sum_across_halves(l_run);
-    const float l_safe = (l_tot == 0.f) ? 1.f : l_tot;
-    const float inv = 1.f / l_safe;
-    const bool valid = q_pos < seq_len;
-    const bool in_t = q_pos < p.T;
-    if (in_t) {
-        ET* orow = obase + (int64_t)q_pos * p.so.t;
-        store_row_transposed<E, D>(orow, o, inv, valid, h);
-        if (lse_base != nullptr && h == 0)
-            lse_base[q_pos] = valid ? (l_tot == 0.f ? -INFINITY : m0 + __log2f(l_tot)) : 0.f;
-    }
-    // a row that sees keys must end with a sum inside the range (a NaN fails the comparison too)
-    const bool bad = (vis.lo <= vis.hi) && (over || !(l_tot >= Lim::kLo && l_tot <= Lim::kHi));
-    return __builtin_amdgcn_ballot_w64(bad) != 0;
+#undef CHILL_STAMP
 }
 
 }  // namespace chill

@@ -418,31 +418,6 @@ constexpr int fwd_lds_bytes() {
     return NS * FwdLds<E, D, TK>::STAGE_BYTES + (fwd_is_fast<E, D, TK, NS>() ? kFwdFastFlagBytes : 0);
 }
 
-// true if `mine` is true for any wave of the workgroup; flags = one int per wave in LDS
-template <int NW>
-__device__ __forceinline__ bool workgroup_any(bool mine, char* flags) {
-    volatile int* f = reinterpret_cast<volatile int*>(flags);
-    if ((threadIdx.x & 63) == 0) f[threadIdx.x >> 6] = mine ? 1 : 0;
-    __syncthreads();
-    int any = 0;
-#pragma unroll
-    for (int w = 0; w < NW; w++) any |= f[w];
-    __syncthreads();  // the flags and the ring are reused
-    return any != 0;
-}
-
-template <typename E, int D, int MASK, int NW, int TK, int NS>
-__device__ __forceinline__ void fwd_one_q_tile(const FwdParams& p, char* smem, int b, int hd, int qt,
-                                               int wave_has_full_blocks) {
-    if constexpr (fwd_is_fast<E, D, TK, NS>()) {
-        const bool again = fwd_q_tile_fast<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt);
-        if (workgroup_any<NW>(again, smem + NS * FwdLds<E, D, TK>::STAGE_BYTES))
-            fwd_q_tile<E, D, MASK, NW, TK, 3>(p, smem, b, hd, qt, wave_has_full_blocks);
-    } else {
-        fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt, wave_has_full_blocks);
-    }
-}
-
 // Workgroups of four waves whose LDS ring leaves room for a second workgroup on the CU are compiled
 // for 256 registers per wave, so that two of them share a CU: one computes while the other loads its
 // first tiles or stores its result.
@@ -469,10 +444,15 @@ void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
     const int b = bh / p.H;
     const int hd = bh % p.H;
     const int qt_hi = n_q_tiles - 1 - j;
-    fwd_one_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, wave_has_full_blocks);
-    if (paired && j != qt_hi) {
-        __syncthreads();  // the LDS ring is reused
-        fwd_one_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
+    if constexpr (fwd_is_fast<E, D, TK, NS>()) {
+        fwd_fast_q_tiles<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, (paired && j != qt_hi) ? j : -1,
+                                                 wave_has_full_blocks);
+    } else {
+        fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, qt_hi, wave_has_full_blocks);
+        if (paired && j != qt_hi) {
+            __syncthreads();  // the LDS ring is reused
+            fwd_q_tile<E, D, MASK, NW, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
+        }
     }
 }
 

@@ -14,8 +14,10 @@ rotation in front of the first one to the last O^T += V^T P^T:
     fill                          S(g), S(g+1) and P(g) of the first tile; V operands of step g
     while cnt > 1:  step 0, step 1, cnt -= 1, ring_top
     drain                         the two steps of the last tile without looking ahead
-    (ring_top: wait for the tile ahead, barrier, rotate the ring, issue a new tile; the caller does it
-    for the first tile)
+ring_top = wait for the tile ahead, barrier, rotate the ring, issue a new tile.  The caller does the
+first one except for the issue.  While tiles remain to be issued, the scalar work of ring_top rides in
+the slots of the steps (the loads of the tile under step 0, the rotation under step 1) and only the
+wait and the barrier stand between two tiles.
 
 Step g of the loop (parity PAR = g & 1), 2 * NS slots (NS = D / 16):
   matrix pipe   slots 0 .. NS-1:   O^T[db] += V(g)^T P(g)^T
@@ -253,7 +255,9 @@ def wait_lgkm(st: Stream, n: int):
     st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
 
 
-def gen_step(c: Config, st: Stream, par: int):
+def gen_step(c: Config, st: Stream, par: int, filler=(), late_filler=()):
+    """One step.  `filler`: closures (scalar work: ring rotation, tile loads) dealt over all slots;
+    `late_filler`: closures dealt over the slots of the second phase only."""
     NS = c.NS
     ops = softmax_ops(c, st, c.S[par ^ 1], c.P[par ^ 1])
     nslots = 2 * NS
@@ -261,24 +265,77 @@ def gen_step(c: Config, st: Stream, par: int):
     share = [0] * nslots
     for t in range(1, nslots):
         share[t] = len(ops) * t // (nslots - 1) - len(ops) * (t - 1) // (nslots - 1)
-    it = iter(ops)
+    fshare = [len(filler) * (t + 1) // nslots - len(filler) * t // nslots for t in range(nslots)]
+    lshare = [0] * NS + [len(late_filler) * (t + 1) // NS - len(late_filler) * t // NS for t in range(NS)]
+    it, fit, lit = iter(ops), iter(filler), iter(late_filler)
+
+    def fill_slot(t):
+        for _ in range(share[t]):
+            next(it)()
+        for _ in range(fshare[t]):
+            next(fit)()
+        for _ in range(lshare[t]):
+            next(lit)()
+
     for t in range(NS):
         # LDS reads issued after V operand t: V t+1 .. NS-1 (2 each), then K 0 .. t-1
         wait_lgkm(st, 2 * (NS - 1 - t) + t)
         mfma_pv(c, st, t, c.P[par])
         read_k(c, st, t, c.KA, par)                       # K of step g+2: block `par` of the next tile
-        for _ in range(share[t]):
-            next(it)()
+        fill_slot(t)
     for t in range(NS):
         # LDS reads issued after K operand t: K t+1 .. NS-1, then V 0 .. t-1 (2 each)
         wait_lgkm(st, (NS - 1 - t) + 2 * t)
         mfma_qk(c, st, t, c.S[par])
         # V of step g+1: block 1 of this tile (par = 0) or block 0 of the next (par = 1)
         read_v(c, st, t, c.VA[par], par ^ 1)
-        for _ in range(share[NS + t]):
-            next(it)()
-    assert next(it, None) is None
+        fill_slot(NS + t)
+    assert next(it, None) is None and next(fit, None) is None and next(lit, None) is None
     block_sum_check(c, st)
+
+
+def issue_ops(c: Config, st: Stream):
+    """The loads of one tile into the stage at `tfill` (tm0 = tfill + wave * 1024), as closures of one
+    load each: K slabs j * NW + wave, then V slabs.  A wave without a slab in the last round runs that
+    load with an empty EXEC (no branches: these closures are dealt over the slots of a step)."""
+    ops = []
+    A = st.add
+    for kind, per, slabs, base, gbase, ptr in (("k", c.kper, c.kslabs, 0, c.GK, "kb"),
+                                              ("v", c.vper, c.vslabs, c.kbytes, c.GV, "vb")):
+        for j in range(per):
+            partial = (j + 1) * c.NW > slabs
+
+            def load(j=j, partial=partial, base=base, gbase=gbase, ptr=ptr, kind=kind):
+                if partial:
+                    A(f"s_mov_b64 exec, %[{kind}last]", "salu")
+                A(f"s_add_u32 m0, %[tm0], {base + j * c.NW * 1024}", "salu")
+                A("s_nop 0", "nop")
+                A(f"global_load_lds_dwordx4 {vr(gbase + j)}, s[{PTR_SGPR[ptr]}:{PTR_SGPR[ptr] + 1}]", "vmem", [gbase + j])
+                if partial:
+                    A("s_mov_b64 exec, -1", "salu")
+            ops.append(load)
+        lo, hi = f"s{PTR_SGPR[ptr]}", f"s{PTR_SGPR[ptr] + 1}"
+
+        def advance(lo=lo, hi=hi, kind=kind):
+            A(f"s_add_u32 {lo}, {lo}, %[{kind}step]", "salu")
+            A(f"s_addc_u32 {hi}, {hi}, 0", "salu")
+        ops.append(advance)
+    return ops
+
+
+def rotate_ops(c: Config, st: Stream):
+    """The ring moves on by one tile (scalar part), as closures for the slots of a step."""
+    A = st.add
+    return [
+        lambda: A("s_mov_b32 %[tfill], %[cur]", "salu"),
+        lambda: A("s_mov_b32 %[cur], %[tnext]", "salu"),
+        lambda: A(f"s_add_u32 %[tnext], %[tnext], {c.stage}", "salu"),
+        lambda: A("s_cmp_eq_u32 %[tnext], %[ringend]", "salu"),
+        lambda: A("s_cselect_b32 %[tnext], %[lds0], %[tnext]", "salu"),
+        lambda: A("s_add_u32 %[tm0], %[tfill], %[w1024]", "salu"),
+        lambda: A("s_sub_i32 %[rem], %[rem], 1", "salu"),
+        lambda: A("s_sub_i32 %[cnt], %[cnt], 1", "salu"),
+    ]
 
 
 def gen_ring_top(c: Config, st: Stream, tag: str):
@@ -305,6 +362,8 @@ def gen_ring_top(c: Config, st: Stream, tag: str):
     A("s_cmp_eq_u32 %[tnext], %[ringend]", "salu")
     A("s_cselect_b32 %[tnext], %[lds0], %[tnext]", "salu")
     A(f"s_cmp_gt_i32 %[rem], {c.FL}", "salu")
+    if "noissue" in c.ablate:
+        A(f"s_branch .Lnoissue{tag}%=", "salu")
     A(f"s_cbranch_scc0 .Lnoissue{tag}%=", "salu")
     # K slabs j * NW + wave, then V slabs; the last round only for the waves whose slab exists
     A("s_add_u32 %[tm0], %[tfill], %[w1024]", "salu")
@@ -374,40 +433,85 @@ def gen_drain(c: Config, st: Stream):
     st.add("s_nop 7", "nop", nops=8)
 
 
+def gen_issue_now(c: Config, st: Stream):
+    for op in issue_ops(c, st):
+        op()
+    st.add("s_sub_i32 %[rem], %[rem], 1", "salu")
+
+
 def gen_loop(c: Config):
     def S():
         return Stream()
 
-    head, fill, steps, top, drain = S(), S(), S(), S(), S()
+    head, fill, fast, steps, top, drain, pre_drain = S(), S(), S(), S(), S(), S(), S()
     # operands that the compiler produced with vector instructions settle first
     head.add("s_nop 4", "nop", nops=5)
     head.add(f"s_add_u32 %[ringend], %[lds0], {c.NSTG * c.stage}", "salu")
-    # the caller has rotated the ring for the first tile: `cur` is its stage
+    # The caller has waited, synchronised and rotated for the first tile (`cur` is its stage) but not
+    # issued the tile that goes to the stage freed by that (`tfill`): that load is pending.
     head.add(f"s_add_u32 %[tnext], %[cur], {c.stage}", "salu")
     head.add("s_cmp_eq_u32 %[tnext], %[ringend]", "salu")
     head.add("s_cselect_b32 %[tnext], %[lds0], %[tnext]", "salu")
+    head.add(f"s_sub_u32 %[tfill], %[cur], {c.stage}", "salu")
+    head.add("s_cmp_eq_u32 %[cur], %[lds0]", "salu")
+    head.add(f"s_cselect_b32 %[tfill], {(c.NSTG - 1) * c.stage}, %[tfill]", "salu")
+    head.add("s_cselect_b32 %[tm0], %[lds0], 0", "salu")
+    head.add("s_add_u32 %[tfill], %[tfill], %[tm0]", "salu")
+    head.add("s_add_u32 %[tm0], %[tfill], %[w1024]", "salu")
     head.add(f"v_add_u32 {vr(c.KA)}, %[tnext], {vr(c.KLANE)}", "valu", [c.KLANE], [c.KA])
     head.add(f"v_add_u32 {vr(c.VA[0])}, %[cur], {vr(c.VLANE)}", "valu", [c.VLANE], [c.VA[0]])
     head.add(f"v_add_u32 {vr(c.VA[1])}, %[tnext], {vr(c.VLANE)}", "valu", [c.VLANE], [c.VA[1]])
+    # EXEC of the loads of the last round: all lanes for the waves that have a slab in it
+    head.add(f"s_cmp_lt_u32 %[wave], {c.kslabs - (c.kper - 1) * c.NW}", "salu")
+    head.add("s_cselect_b64 %[klast], -1, 0", "salu")
+    head.add(f"s_cmp_lt_u32 %[wave], {c.vslabs - (c.vper - 1) * c.NW}", "salu")
+    head.add("s_cselect_b64 %[vlast], -1, 0", "salu")
     gen_fill(c, fill)
+    # fast tile: the pending loads under step 0, the rotation under step 1 (the K address of the next
+    # tile behind the last K read of step 1), then only the wait and the barrier between tiles
+    gen_step(c, fast, 0, filler=issue_ops(c, fast))
+    gen_step(c, fast, 1, filler=rotate_ops(c, fast),
+             late_filler=[lambda: fast.add(f"v_add_u32 {vr(c.KA)}, %[tnext], {vr(c.KLANE)}", "valu", [c.KLANE], [c.KA])])
+    fast.add(f"s_waitcnt vmcnt({c.FL * c.loads_min})", "wait")
+    if "barrier" not in c.ablate:
+        fast.add("s_barrier", "salu")
+    fast.add(f"v_mov_b32 {vr(c.VA[0])}, {vr(c.VA[1])}", "valu", [c.VA[1]], [c.VA[0]])
+    fast.add(f"v_add_u32 {vr(c.VA[1])}, %[tnext], {vr(c.VLANE)}", "valu", [c.VLANE], [c.VA[1]])
     gen_step(c, steps, 0)
     gen_step(c, steps, 1)
     gen_ring_top(c, top, "")
+    gen_issue_now(c, pre_drain)
     gen_drain(c, drain)
-    # what can follow what: fill -> drain; fill -> (steps -> ring_top)+ -> drain
+    # what can follow what
     if not c.ablate:
-        check_stream(head.ins + fill.ins + drain.ins, c.name + " (one tile)")
-        check_stream(head.ins + fill.ins + steps.ins + top.ins + steps.ins + top.ins + steps.ins + top.ins + drain.ins,
-                     c.name)
+        check_stream(head.ins + fill.ins + pre_drain.ins + drain.ins, c.name + " (one tile)")
+        check_stream(head.ins + fill.ins + fast.ins + fast.ins + fast.ins + pre_drain.ins + drain.ins, c.name + " (fast)")
+        check_stream(head.ins + fill.ins + fast.ins + fast.ins + steps.ins + top.ins + steps.ins + top.ins + drain.ins,
+                     c.name + " (fast, then the last tiles)")
     out = S()
     out.ins += head.ins + fill.ins
-    out.add(".Lcheck%=:", "label", nops=0)
+    # fast tiles while a load is pending and a tile follows
+    out.add(".Lfast%=:", "label", nops=0)
+    out.add("s_cmp_le_i32 %[cnt], 1", "salu")
+    out.add("s_cbranch_scc1 .Lpredrain%=", "salu")
+    out.add(f"s_cmp_le_i32 %[rem], {c.FL}", "salu")
+    out.add("s_cbranch_scc1 .Lrest%=", "salu")
+    out.ins += fast.ins
+    out.add("s_branch .Lfast%=", "salu")
+    # the last tile of the statement is next: the pending load, if there is one
+    out.add(".Lpredrain%=:", "label", nops=0)
+    out.add(f"s_cmp_le_i32 %[rem], {c.FL}", "salu")
+    out.add("s_cbranch_scc1 .Ldrain%=", "salu")
+    out.ins += pre_drain.ins
+    out.add("s_branch .Ldrain%=", "salu")
+    # nothing left to load: plain steps, then the wait, the barrier and the rotation
+    out.add(".Lrest%=:", "label", nops=0)
     out.add("s_cmp_le_i32 %[cnt], 1", "salu")
     out.add("s_cbranch_scc1 .Ldrain%=", "salu")
     out.ins += steps.ins
     out.add("s_sub_i32 %[cnt], %[cnt], 1", "salu")
     out.ins += top.ins
-    out.add("s_branch .Lcheck%=", "salu")
+    out.add("s_branch .Lrest%=", "salu")
     out.add(".Ldrain%=:", "label", nops=0)
     out.ins += drain.ins
     return out.ins
@@ -424,7 +528,7 @@ def operand_lists(c: Config):
         outs.append((n, f"+{{s[{PTR_SGPR[n]}:{PTR_SGPR[n] + 1}]}}"))
     if c.elem == "f16":
         outs.append(("over", "+s"))
-    for n in ("tfill", "tnext", "tm0", "ringend"):
+    for n in ("tfill", "tnext", "tm0", "ringend", "klast", "vlast"):
         outs.append((n, "=&s"))
     nq = 4 * c.NS
     for i in range(0, nq, 16):
@@ -452,15 +556,15 @@ def operand_lists(c: Config):
 def emit_macro(c: Config, out):
     ins = gen_loop(c)
     outs, inputs, clob = operand_lists(c)
-    temps = ("tfill", "tnext", "tm0", "ringend")
+    temps = ("tfill", "tnext", "tm0", "ringend", "klast", "vlast")
     names = [n for n, _ in outs if n not in temps] + [n for n, _ in inputs]
     out.write(f"// {c.name}: {c.elem} D={c.D}, {c.NW} waves, {c.NSTG} stages; {c.nvgpr} vector registers\n")
     out.write(f"#define {c.name}_VGPRS {c.nvgpr}\n")
     out.write(f"#define {c.name}({', '.join('A_' + n for n in names)}) \\\n")
-    out.write("    do { unsigned t_fill_, t_next_, t_m0_, t_end_; asm volatile( \\\n")
+    out.write("    do { unsigned t_fill_, t_next_, t_m0_, t_end_; unsigned long long t_kl_, t_vl_; asm volatile( \\\n")
     for i in ins:
         out.write(f'        "{i["text"]}\\n\\t" \\\n')
-    tmpmap = {"tfill": "t_fill_", "tnext": "t_next_", "tm0": "t_m0_", "ringend": "t_end_"}
+    tmpmap = {"tfill": "t_fill_", "tnext": "t_next_", "tm0": "t_m0_", "ringend": "t_end_", "klast": "t_kl_", "vlast": "t_vl_"}
     o_s = ", ".join(f'[{n}] "{cs}"({tmpmap.get(n, "A_" + n)})' for n, cs in outs)
     i_s = ", ".join(f'[{n}] "{cs}"(A_{n})' for n, cs in inputs)
     c_s = ", ".join(f'"{x}"' for x in ["memory", "vcc", "scc"] + clob)
