@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import ctypes
 import logging
+import math
 import typing
 
 import torch
@@ -41,18 +42,30 @@ def _stream_ptr(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def _check_inputs(q, k, v, lens, sm_scale):
-    assert q.ndim == 4 and k.ndim == 4 and v.ndim == 4, "q, k, v must be [B, H, T, D]"
+def _require(cond: bool, message: str):
+    # explicit raises: input validation must survive ``python -O``
+    if not cond:
+        raise ValueError(f"chill_attention: {message}")
+
+
+def _check_inputs(q, k, v, lens, sm_scale, others=()):
+    """Shapes, dtypes and devices of one call; ``others`` = further tensors (o, lse, do) that must live
+    on q's device.  Everything the kernels dereference is checked here: a tensor on the CPU or on
+    another GPU would reach them as a bad pointer."""
+    _require(q.ndim == 4 and k.ndim == 4 and v.ndim == 4, "q, k, v must be [B, H, T, D]")
     batch, heads, T, head_dim = q.shape
     num_kv_heads = k.shape[1]
-    assert heads % num_kv_heads == 0
-    assert head_dim in _HEAD_DIMS
-    assert head_dim == k.shape[-1] and head_dim == v.shape[-1]
-    assert T == k.shape[-2] and T == v.shape[-2]
-    assert k.shape[0] == batch and v.shape[0] == batch and v.shape[1] == num_kv_heads
-    assert q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype
-    assert sm_scale is not None
-    assert lens is None or (lens.dtype == torch.int32 and batch == len(lens) and lens.ndim == 1)
+    _require(heads % num_kv_heads == 0, "the number of query heads must be a multiple of the key/value heads")
+    _require(head_dim in _HEAD_DIMS, f"head dim must be one of {_HEAD_DIMS}")
+    _require(head_dim == k.shape[-1] and head_dim == v.shape[-1], "q, k, v must share the head dim")
+    _require(T == k.shape[-2] and T == v.shape[-2], "q, k, v must share the sequence length")
+    _require(k.shape[0] == batch and v.shape[0] == batch and v.shape[1] == num_kv_heads, "batch / head mismatch")
+    _require(q.dtype in _DTYPES and k.dtype == q.dtype and v.dtype == q.dtype, "q, k, v must share a dtype of fp32 / fp16 / bf16")
+    _require(sm_scale is not None and math.isfinite(float(sm_scale)), "sm_scale must be a finite number")
+    _require(lens is None or (lens.dtype == torch.int32 and lens.ndim == 1 and batch == len(lens)),
+             "lens must be an int32 vector with one entry per batch element")
+    for name, t in (("k", k), ("v", v), ("lens", lens)) + tuple(others):
+        _require(t is None or t.device == q.device, f"{name} is on {t.device if t is not None else None}, q on {q.device}")
     if not q.is_cuda:
         raise RuntimeError("chill_attention runs on the GPU only (tensors must be on a ROCm 'cuda' device)")
 
@@ -149,7 +162,8 @@ def register_chill_mask(mask: ChillMask):
         precision: str,
         autotune: bool,
     ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-        _check_inputs(q, k, v, lens, sm_scale)
+        _check_inputs(q, k, v, lens, sm_scale, others=(("o", o), ("lse", lse), ("do", do)))
+        _require(o.shape == q.shape and do.shape == q.shape and lse.shape == q.shape[:3], "o, do, lse must match q")
         batch, heads, T, head_dim = q.shape
         num_kv_heads = k.shape[1]
         desc = mask_cls_descriptor(mask_args)

@@ -44,11 +44,9 @@ class ChillMask(ABC):
     def __init__(self, constargs=None):
         self.constargs = constargs or tuple()
         self.name = type(self).__name__
-        assert isinstance(self.constargs, tuple), "As of now, only tuple can be passed as args"
+        assert isinstance(self.constargs, tuple), "mask arguments are given as one tuple"
         for i in self.constargs:
-            assert isinstance(
-                i, (int, float, bool)
-            ), "Pytorch interface only supports typing.Union[int, float, bool] parametrization"
+            assert isinstance(i, (int, float, bool)), "a mask argument must be an int, a float or a bool (operator schema)"
 
     def __str__(self):
         return f"{self.name}({', '.join(map(str, self.constargs))})"

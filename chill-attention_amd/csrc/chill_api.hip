@@ -52,6 +52,18 @@ static int check_dtype_dim(int dtype, int D, int* es) {
     return CHILL_OK;
 }
 
+// The exponent's factor sm_scale * log2(e).  The kernels multiply it into raw scores of which the
+// masked ones are -inf, so it must not be zero: a zero scale (uniform attention over the visible keys,
+// chill_fwd.py:213-214 scales first and masks afterwards) becomes one so small that every finite score
+// still rounds to exponent 0.  Non-finite scales are refused.
+static int lower_scale(float sm_scale, float* scale_log2) {
+    if (!(sm_scale - sm_scale == 0.f)) return CHILL_ERR_BAD_ARGUMENT;
+    float s = sm_scale * 1.4426950408889634f;
+    if (s == 0.f) s = 1e-30f;
+    *scale_log2 = s;
+    return CHILL_OK;
+}
+
 static int check_shape(int B, int H, int H_kv, int T) {
     if (B <= 0 || H <= 0 || H_kv <= 0 || T <= 0) return CHILL_ERR_BAD_SHAPE;
     if (H % H_kv != 0) return CHILL_ERR_BAD_SHAPE;
@@ -122,7 +134,7 @@ int chill_fwd(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* 
     p.H_kv = H_kv;
     p.T = T;
     p.group = H / H_kv;
-    p.scale_log2 = sm_scale * 1.4426950408889634f;
+    CHILL_TRY(lower_scale(sm_scale, &p.scale_log2));
     return kFwd[dtype][dim_index(D)](p, mask->id, static_cast<hipStream_t>(stream));
 }
 
@@ -174,7 +186,7 @@ static int lower_bwd(BwdParams* p, const ChillTensor4* q, const ChillTensor4* k,
     p->T = T;
     p->group = H / H_kv;
     p->sm_scale = sm_scale;
-    p->scale_log2 = sm_scale * 1.4426950408889634f;
+    CHILL_TRY(lower_scale(sm_scale, &p->scale_log2));
     return CHILL_OK;
 }
 

@@ -157,6 +157,30 @@ def test_cpu_tensors_are_refused():
         ca.chill_attention(q, q, q, mask=ca.CausalChillMask())
 
 
+def test_inputs_on_other_devices_are_refused_before_any_launch():
+    """A k, v, lens, o, lse or dO that does not live on q's device would reach the kernels as a bad
+    pointer: the adapters refuse it (checked here without a GPU, on the validation function)."""
+    import torch
+
+    from chill_attention import chill
+
+    q = torch.empty(2, 2, 16, 16, device="meta")
+    cpu = torch.zeros(2, 2, 16, 16)
+    with pytest.raises(ValueError, match="k is on cpu"):
+        chill._check_inputs(q, cpu, q, None, 1.0)
+    with pytest.raises(ValueError, match="lens is on cpu"):
+        chill._check_inputs(q, q, q, torch.ones(2, dtype=torch.int32), 1.0)
+    with pytest.raises(ValueError, match="do is on cpu"):
+        chill._check_inputs(q, q, q, None, 1.0, others=(("o", q), ("do", cpu)))
+    with pytest.raises(ValueError, match="finite"):
+        chill._check_inputs(q, q, q, None, float("nan"))
+    with pytest.raises(ValueError, match="head dim"):
+        bad = torch.empty(2, 2, 16, 24, device="meta")
+        chill._check_inputs(bad, bad, bad, None, 1.0)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        chill._check_inputs(cpu, cpu, cpu, None, 1.0)
+
+
 def test_tile_sweep_candidates():
     """The sweep tool's candidate list: the shipped shape comes first and overrides nothing."""
     from chill_attention import tune

@@ -2,12 +2,14 @@
 
 Inputs follow the benchmark protocol: q, k, v, dO drawn in that order from
 torch.Generator('cpu').manual_seed(seed) as fp32 N(0, sigma), cast to the config dtype.  Checked
-  * against the oracle (dense mask -> torch SDPA + autograd on fp32-upcast inputs) on head slices the
-    oracle finishes in seconds, with the tolerance of the benchmark definition:
-    atol = rtol = 1e-2 for bf16 / fp16, 1e-4 for fp32 (O, dQ, dK, dV);
+  * against the oracle (dense mask -> torch SDPA + autograd on fp32-upcast inputs) on eight (batch, head)
+    slices per configuration (every one for the small ones), spread over the work-item order of the
+    launch (first, last and middle items of the runs the eight XCDs get), with the tolerance of the
+    benchmark definition: atol = rtol = 1e-2 for bf16 / fp16, 1e-4 for fp32 (O, dQ, dK, dV); the largest
+    errors are printed;
   * through size-independent properties on the full outputs: V = 1 gives O = 1 (rows of P sum to 1),
-    O stays inside [min V, max V], sum(dQ*Q) == sum(dK*K), and any (batch, head) slice run alone
-    reproduces the full run bit for bit.
+    O stays inside [min V, max V], sum(dQ*Q) == sum(dK*K), and a (batch, head) slice run alone stays
+    within the same tolerance (bit for bit where the slice's launch uses the same tile shape).
 """
 
 import json
@@ -25,6 +27,24 @@ with open(os.path.join(os.path.dirname(__file__), "golden", "baseline_configs.js
     CONFIGS = {c["name"]: c for c in json.load(f)["configs"]}
 DT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
 TOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 1e-2}
+
+
+def oracle_slices(B, H):
+    """(batch, head) pairs for the oracle.  Work items are (batch * H + head) * tiles + tile, dealt to
+    the 8 XCDs in contiguous runs: the first and the last item, items on both sides of XCD run
+    boundaries, and some from the middle of runs."""
+    n = B * H
+    if n <= 8:
+        return [(i // H, i % H) for i in range(n)]
+    per = -(-n // 8)
+    picks = {0, n - 1, per - 1, per, 3 * per + per // 2, 4 * per - 1, 4 * per, 6 * per + 1}
+    return [(i // H, i % H) for i in sorted(min(max(i, 0), n - 1) for i in picks)]
+
+
+def report(name, what, got, want):
+    diff = (got.float() - want.float()).abs()
+    rel = (diff / want.float().abs().clamp_min(1e-3)).max().item()
+    print(f"  {name} {what}: max abs err {diff.max().item():.3e}, max rel err (|want| >= 1e-3) {rel:.3e}", flush=True)
 
 
 def inputs(c):
@@ -51,20 +71,33 @@ def test_baseline_config(name):
     assert torch.isfinite(out).all() and torch.isfinite(lse).all()
 
     # oracle on a few (batch, head) slices
-    slices = [(0, 0), (c["B"] - 1, c["H"] - 1)] if c["T"] > 4096 else [(b, h) for b in range(min(c["B"], 2)) for h in range(min(c["H"], 4))]
+    from chill_attention import _lib
+    from chill_attention.tiles import tile_config
+
+    slices = oracle_slices(c["B"], c["H"])
+    assert len(slices) >= min(8, c["B"] * c["H"])
     for b, h in slices:
         qs, ks, vs = (x.detach()[b : b + 1, h : h + 1].float().clone().requires_grad_(not fwd_only) for x in (q, k, v))
         ref, _ = orc.reference_naive(c["mask"], tuple(c["args"]), qs, ks, vs, None)
+        report(name, f"slice {(b, h)} O", out.detach()[b : b + 1, h : h + 1], ref.detach().to(dtype))
         torch.testing.assert_close(out.detach()[b : b + 1, h : h + 1], ref.detach().to(dtype), atol=tol, rtol=tol)
         if not fwd_only:
             ref.backward(do[b : b + 1, h : h + 1].float())
             for nm, got, want in (("dq", q.grad, qs.grad), ("dk", k.grad, ks.grad), ("dv", v.grad, vs.grad)):
+                report(name, f"slice {(b, h)} {nm}", got[b : b + 1, h : h + 1], want.to(dtype))
                 torch.testing.assert_close(got[b : b + 1, h : h + 1], want.to(dtype), atol=tol, rtol=tol, msg=lambda s: f"{name} {nm} slice {(b, h)}: {s}")
         del ref, qs, ks, vs
-        # a slice run on its own is the same computation: bit-identical
+    # a slice run on its own is the same computation: within the tolerance always, and bit-identical when
+    # its launch takes the same row of the tile table (small launches take the short-sequence row)
+    for b, h in (slices[0], slices[-1]):
         with torch.no_grad():
             alone = ca.chill_attention(q.detach()[b : b + 1, h : h + 1], k.detach()[b : b + 1, h : h + 1], v.detach()[b : b + 1, h : h + 1], mask=mask)
-        assert torch.equal(alone, out.detach()[b : b + 1, h : h + 1])
+        full = out.detach()[b : b + 1, h : h + 1]
+        torch.testing.assert_close(alone, full, atol=tol, rtol=tol)
+        same_shape = (tile_config(mask, c["D"], dtype, _lib.PASS_FWD, seq_len=c["T"], batch_heads=1)
+                      == tile_config(mask, c["D"], dtype, _lib.PASS_FWD, seq_len=c["T"], batch_heads=c["B"] * c["H"]))
+        if same_shape:
+            assert torch.equal(alone, full)
 
     # properties on the full tensors
     with torch.no_grad():
