@@ -33,14 +33,73 @@ PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}  # MI355X dense MFMA
 PEAK_HBM_GBS = 8000.0
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), scaled by what
-# the same counters read for a plain 1 GiB copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000);
-# the summaries of those runs are kept under profiles/.  (workload, kernel) -> bytes
+# the same counters read for a plain 1 GiB copy in the same run (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
+# The figures come from the summary named in TRAFFIC_SOURCE, which records the digest of the kernel
+# sources it was measured on (kernel_sources_digest below); with other sources the line reports null.
+TRAFFIC_SOURCE = "profiles/c3_causal_bf16_fwd_bwd_kernels.md"
 MEASURED_TRAFFIC = {
     ("C3", "chill_fwd"): (696510 * 2.0 + 266243) * 1024,
     ("C3", "chill_bwd_delta"): (262171 * 2.0 + 4193) * 1024,
     ("C3", "chill_bwd_dkdv"): (534807 * 2.0 + 540102) * 1024,
     ("C3", "chill_bwd_dq"): (747358 * 2.0 + 262144) * 1024,
 }
+
+
+def kernel_sources_digest():
+    """sha1 over the kernel sources (csrc/*.h, *.hip, *.cpp, *.py, Makefile): names the build a profile
+    summary belongs to."""
+    import hashlib
+
+    csrc = os.path.join(ROOT, "chill-attention_amd", "csrc")
+    h = hashlib.sha1()
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".h", ".hip", ".cpp", ".py")) or name == "Makefile":
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:12]
+
+
+def traffic_is_current():
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_SOURCE)) as f:
+            return f"kernel sources digest: {kernel_sources_digest()}" in f.read()
+    except OSError:
+        return False
+
+
+class ClockSampler:
+    """Shader clock (MHz) while the GPU works, as `rocm-smi --showclocks` reports it, sampled from a thread."""
+
+    def __init__(self, period_s=0.4):
+        import threading
+
+        self.samples, self.period, self._stop = [], period_s, threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        import re
+        import subprocess
+
+        while not self._stop.is_set():
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+                m = re.search(r"sclk clock level[^\n]*\((\d+)Mhz\)", out)
+                if m:
+                    self.samples.append(int(m.group(1)))
+            except Exception:
+                return
+            self._stop.wait(self.period)
+
+    def __enter__(self):
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join(timeout=15)
+
+    def mean(self):
+        return sum(self.samples) / len(self.samples) if self.samples else None
 
 # name -> (mask ctor name, args, dtype, B, H, T, D, seed, sigma)
 WORKLOADS = {
@@ -172,6 +231,8 @@ def main():
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--mode", default="fwd+bwd", choices=["fwd", "fwd+bwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sustained-seconds", type=float, default=3.0,
+                    help="length of the continuous loop behind the `sustained` figure (0: leave it out)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain 1 GiB device copy (1 GiB read + 1 GiB written) before the warm-up: "
                          "the known-size dispatch that scales the FETCH_SIZE / WRITE_SIZE counters of a "
@@ -234,6 +295,43 @@ def main():
     value = step_flops / (ms_per_step * 1e-3) / 1e12
     peak = PEAK_TFLOPS[dname]
 
+    # The timed region above is short (the board has not settled at its power limit yet).  `sustained`: the
+    # same launches in one continuous loop of a few seconds, with the shader clock sampled meanwhile.
+    sustained = None
+    if args.sustained_seconds > 0:
+        n_loop = max(int(args.sustained_seconds / (ms_per_step * 1e-3)), args.steps)
+        with ClockSampler() as clock:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n_loop):
+                for _, fn in kernels:
+                    fn()
+            torch.cuda.synchronize()
+            loop_s = time.perf_counter() - t0
+        sustained = {"value": step_flops * n_loop / loop_s / 1e12, "unit": "TFLOP/s", "steps": n_loop,
+                     "seconds": loop_s, "ms_per_step": loop_s * 1e3 / n_loop, "sm_clock_mhz": clock.mean(),
+                     "frac_of_peak": step_flops * n_loop / loop_s / 1e12 / peak}
+
+    # the same step through the public operator (chill_attention + autograd): allocation and dispatch included
+    op_ms = None
+    if args.sustained_seconds > 0:
+        qa, ka, va = (x.detach().clone().requires_grad_(mode == "fwd+bwd") for x in (q, k, v))
+
+        def op_step():
+            o = ca.chill_attention(qa, ka, va, mask=mask)
+            if mode == "fwd+bwd":
+                o.backward(do)
+                qa.grad = ka.grad = va.grad = None
+
+        for _ in range(3):
+            op_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            op_step()
+        torch.cuda.synchronize()
+        op_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
     # algorithmic FLOPs per launch: forward 4*D per unmasked entry (2 GEMMs); of the backward's
     # 10*D (5 GEMMs: S, dP, dV, dK, dQ) the dK/dV kernel is charged S, dP, dV, dK = 8*D and the dQ
     # kernel dQ = 2*D (its own S and dP are recomputation, not algorithmic work)
@@ -250,8 +348,10 @@ def main():
         roof = {"kernel": dom_name, "bound": "mfma", "achieved": alg / (k_ms[dom] * 1e-3) / 1e12, "peak": peak,
                 "unit": "TFLOP/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, dom_name))
+    current = traffic_is_current()
+    roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, dom_name)) if current else None
     roof["traffic_unit"] = "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-scaled)"
+    roof["traffic_source"] = TRAFFIC_SOURCE if current else f"none: {TRAFFIC_SOURCE} was measured on other kernel sources"
     roof["algorithmic_bytes"] = {
         "chill_fwd": 4.0 * B * H * T * D * es + 4.0 * B * H * T,
         "chill_bwd_delta": 2.0 * B * H * T * D * es + 4.0 * B * H * T,
@@ -282,6 +382,10 @@ def main():
         "fwd_tflops": fwd_flops / (k_ms[0] * 1e-3) / 1e12,
         "fwd_frac_of_peak": fwd_flops / (k_ms[0] * 1e-3) / 1e12 / peak,
         "roofline": roof,
+        "sustained": sustained,
+        "sm_clock_mhz": sustained["sm_clock_mhz"] if sustained else None,
+        "operator_ms_per_step": op_ms,
+        "kernel_sources_digest": kernel_sources_digest(),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, mask_name, margs, dname, T, D, mode, seed, sigma)

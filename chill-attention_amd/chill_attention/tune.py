@@ -95,6 +95,22 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
     return rows
 
 
+def check_hand_managed_registers(macros: dict | None = None) -> None:
+    """Raise RuntimeError unless, in every kernel that names accumulation registers itself (16-bit inputs,
+    head dim 256), the compiler stays below the registers the kernel names and spills nothing.  The check
+    reads the assembly hipcc writes for the given build (``macros`` as for the library build); it covers
+    register overlap and spills, nothing else.  Part of every build of the library."""
+    for elem in ("bf16", "f16"):
+        rows = hand_managed_registers(elem, 256, macros)
+        if not rows:
+            raise RuntimeError(f"no hand-managed kernel found for {elem} head dim 256")
+        for name, compiler_max, hand_min, spilled in rows:
+            if compiler_max >= hand_min or spilled:
+                raise RuntimeError(
+                    f"kernel {name}: the compiler uses accumulation registers up to a{compiler_max} (the kernel "
+                    f"manages a{hand_min} and above itself) or spills ({spilled} registers): this build is unsound")
+
+
 def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | None = None) -> list:
     """Kernels that name accumulation registers themselves (fwd_regs_kernel, dq_regs_kernel, dkdv_regs_kernel) rely on the compiler
     keeping out of them.  Compiles the translation units of (elem, dim) to assembly and

@@ -110,18 +110,14 @@ def build(cls, force: bool = False, jobs: int = 8) -> str:
     if res.returncode != 0 or not os.path.exists(path):
         raise RuntimeError(f"{cls.__name__}: building the mask library failed:\n{res.stdout[-4000:]}")
     # the 16-bit head-dim-256 kernels name accumulation registers themselves: make sure the compiler kept
-    # out of them with this functor inlined (see tune.hand_managed_registers)
+    # out of them with this functor inlined
     from . import tune
 
-    for elem in ("bf16", "f16"):
-        for name, compiler_max, hand_min, spilled in tune.hand_managed_registers(
-                elem, 256, {"CHILL_USER_MASK_HEADER": f'"{header}"'}):
-            if compiler_max >= hand_min or spilled:
-                os.remove(path)
-                raise RuntimeError(
-                    f"{cls.__name__}: with this functor the compiler uses accumulation registers "
-                    f"(up to a{compiler_max}) that the head-dim-256 kernels manage themselves, or spills "
-                    f"({spilled}); simplify the functor (kernel {name})")
+    try:
+        tune.check_hand_managed_registers({"CHILL_USER_MASK_HEADER": f'"{header}"'})
+    except RuntimeError as e:
+        os.remove(path)
+        raise RuntimeError(f"{cls.__name__}: simplify the functor: {e}") from e
     # libraries of this class built from older sources (another key) are of no use any more
     for root in (USER_BUILD_DIR, os.path.dirname(os.path.dirname(path))):
         for name in os.listdir(root):

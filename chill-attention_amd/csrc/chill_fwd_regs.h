@@ -304,6 +304,13 @@ __global__ __launch_bounds__(256) void fwd_regs_kernel(FwdParams p, int n_q_tile
         __syncthreads();  // the LDS ring is reused
         fwd_q_tile_regs<E, D, MASK, TK, NS>(p, smem, b, hd, j, wave_has_full_blocks);
     }
+#ifdef CHILL_TEST_UNSOUND_REGISTERS
+    // For the test of the build's register check only: the COMPILER reads an accumulation register here,
+    // which a kernel that manages a128..a255 by itself must never let happen.
+    float from_accumulation_register;
+    asm volatile("v_accvgpr_write_b32 %0, 0" : "=a"(from_accumulation_register));
+    if (p.lse != nullptr && p.T < 0) p.lse[0] = from_accumulation_register;
+#endif
 }
 
 }  // namespace chill

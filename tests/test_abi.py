@@ -181,6 +181,25 @@ def test_inputs_on_other_devices_are_refused_before_any_launch():
         chill._check_inputs(cpu, cpu, cpu, None, 1.0)
 
 
+def test_build_refuses_unsound_register_use():
+    """__graft_entry__.build() and user_mask.build() end with tune.check_hand_managed_registers: a build in
+    which the compiler touches the accumulation registers that the head-dim-256 kernels manage themselves
+    is refused (here: a build with a macro that makes it do so on purpose)."""
+    import inspect
+    import shutil
+
+    import __graft_entry__ as entry
+    from chill_attention import tune, user_mask
+
+    assert "check_hand_managed_registers" in inspect.getsource(entry.build)
+    assert "check_hand_managed_registers" in inspect.getsource(user_mask.build)
+    if shutil.which("hipcc") is None:
+        pytest.skip("hipcc not on PATH")
+    tune.check_hand_managed_registers()  # the shipped build is sound
+    with pytest.raises(RuntimeError, match="unsound"):
+        tune.check_hand_managed_registers({"CHILL_TEST_UNSOUND_REGISTERS": 1})
+
+
 def test_tile_sweep_candidates():
     """The sweep tool's candidate list: the shipped shape comes first and overrides nothing."""
     from chill_attention import tune
