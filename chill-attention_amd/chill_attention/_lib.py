@@ -61,6 +61,8 @@ def load_library(path: str) -> ctypes.CDLL:
                                    c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
         "chill_bwd_dkdv": (c_int32, [T4, T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, I64_3, c_void_p, c_int64,
                                      c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
+        "chill_bwd_noalloc": (c_int32, [T4, T4, T4, T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, c_int64,
+                                        c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
         "chill_mask_eval_device": (c_int32, [MD, c_int32, c_void_p, c_void_p]),
         "chill_tile_ranges_device": (c_int32, [MD, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p]),
         "chill_mask_eval": (c_int32, [MD, c_int32, P(c_uint8)]),
@@ -87,12 +89,15 @@ def load_library(path: str) -> ctypes.CDLL:
 
 lib = load_library(LIB_PATH)
 EXPORTED_SYMBOLS = (
-    "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dkdv", "chill_mask_eval_device",
+    "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dkdv", "chill_bwd_noalloc", "chill_mask_eval_device",
     "chill_tile_ranges_device", "chill_mask_eval", "chill_mask_limits", "chill_tile_ranges",
     "chill_mask_is_full_block", "chill_mask_has_full_blocks", "chill_tile_config", "chill_tile_config_for_shape",
     "chill_mask_nnz",
     "chill_status_string", "chill_abi_version", "chill_has_user_mask",
 )
+
+
+BWD_NOALLOC_MAX_ROWS = 4 * 1024 * 1024  # CHILL_BWD_NOALLOC_MAX_ROWS of the header
 
 
 def check(fn: str, status: int) -> int:

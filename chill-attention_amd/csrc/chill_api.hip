@@ -3,6 +3,8 @@
 // kept; every launch goes to the caller's stream.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "chill_mask.h"
 #include "chill_params.h"
 
@@ -220,6 +222,56 @@ int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTens
     p.dk = dk->ptr;
     p.dv = dv->ptr;
     return kDkdv[dtype][dim_index(D)](p, mask->id, static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------------------------------------------
+// The whole backward without a workspace from the caller.  The fp32 delta rows, which chill_bwd_delta
+// writes and the two gradient kernels read, live in a device array of this library: each GPU the
+// library runs on holds its own copy of `scratch` until the process ends.  In host code the array's
+// name is a stand-in, not a device address: the address comes from hipGetSymbolAddress, once per
+// device with that device current, and only that pointer is handed to kernels.
+// ---------------------------------------------------------------------------------------------
+constexpr int64_t kNoAllocMaxRows = (int64_t)CHILL_BWD_NOALLOC_MAX_ROWS;
+static __device__ __align__(256) float scratch[kNoAllocMaxRows];
+
+constexpr int kMaxDevices = 64;
+static float* g_scratch_address[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// the current device's copy of `scratch`
+static int scratch_of_current_device(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return CHILL_ERR_HIP;
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    if (g_scratch_address[dev] == nullptr) {
+        float* ptr = nullptr;
+        if (hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr)
+            return CHILL_ERR_HIP;
+        g_scratch_address[dev] = ptr;
+    }
+    *out = g_scratch_address[dev];
+    return CHILL_OK;
+}
+
+int chill_bwd_noalloc(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+                      const ChillTensor4* o, const ChillTensor4* d_o,
+                      const ChillTensor4* dq, const ChillTensor4* dk, const ChillTensor4* dv,
+                      const float* lse, const int64_t lse_stride[3],
+                      const int32_t* lens, int64_t lens_stride,
+                      int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D,
+                      int32_t dtype, float sm_scale, const ChillMaskDesc* mask, void* stream) {
+    CHILL_TRY(check_shape(B, H, H_kv, T));
+    // delta is [B, H, T] fp32, contiguous, in the library's array: sizes beyond it are refused
+    if ((int64_t)B * H * T > kNoAllocMaxRows) return CHILL_ERR_TOO_LARGE;
+    float* delta = nullptr;
+    CHILL_TRY(scratch_of_current_device(&delta));
+    const int64_t delta_stride[3] = {(int64_t)H * T, (int64_t)T, 1};
+    // every row of delta is written by the first launch before the other two read it: nothing to clear
+    CHILL_TRY(chill_bwd_delta(o, d_o, delta, delta_stride, B, H, T, D, dtype, stream));
+    CHILL_TRY(chill_bwd_dkdv(q, k, v, d_o, dk, dv, lse, lse_stride, delta, delta_stride, lens, lens_stride, B, H,
+                             H_kv, T, D, dtype, sm_scale, mask, stream));
+    return chill_bwd_dq(q, k, v, d_o, dq, lse, lse_stride, delta, delta_stride, lens, lens_stride, B, H, H_kv, T, D,
+                        dtype, sm_scale, mask, stream);
 }
 
 }  // extern "C"

@@ -147,7 +147,7 @@ const char* chill_status_string(int32_t status) {
         case CHILL_ERR_BAD_STRIDE: return "bad stride (inner stride must be 1, strides non-negative, rows 16-byte aligned)";
         case CHILL_ERR_HIP: return "HIP launch failure";
         case CHILL_ERR_BAD_ARGUMENT: return "bad argument";
-        case CHILL_ERR_TOO_LARGE: return "problem too large for 32-bit position arithmetic";
+        case CHILL_ERR_TOO_LARGE: return "problem too large (32-bit position arithmetic, or the fixed array of chill_bwd_noalloc)";
         default: return "unknown status";
     }
 }

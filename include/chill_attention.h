@@ -137,6 +137,24 @@ int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTens
                    int32_t dtype, float sm_scale,
                    const ChillMaskDesc* mask, void* stream);
 
+/* The whole backward (delta, then dK/dV, then dQ, as chill_bwd_delta + chill_bwd_dkdv + chill_bwd_dq with
+ * the same arguments) WITHOUT a delta workspace from the caller.  It has no counterpart in the
+ * reference: it is for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  The fp32 delta rows live in an array inside the library,
+ * CHILL_BWD_NOALLOC_MAX_ROWS floats (16 MiB) that every GPU the library runs on holds until the process
+ * ends; B * H * T beyond that returns CHILL_ERR_TOO_LARGE.  The call allocates and frees nothing.  All
+ * calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race on
+ * it; calls on one stream are ordered and need nothing more. */
+#define CHILL_BWD_NOALLOC_MAX_ROWS (4 * 1024 * 1024)
+int chill_bwd_noalloc(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+                      const ChillTensor4* o, const ChillTensor4* d_o,
+                      const ChillTensor4* dq, const ChillTensor4* dk, const ChillTensor4* dv,
+                      const float* lse, const int64_t lse_stride[3],
+                      const int32_t* lens, int64_t lens_stride,
+                      int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D,
+                      int32_t dtype, float sm_scale,
+                      const ChillMaskDesc* mask, void* stream);
+
 /* Device-side evaluation of the mask functors, used to prove that the code the kernels run
  * agrees bit-for-bit with the host enumeration (the role ChillMask._mask_infer, mask.py:282-330,
  * plays for the Triton functions).  Writes `n*n` bytes (row = q, col = k) of
