@@ -30,7 +30,7 @@ typedef int i32x16 __attribute__((ext_vector_type(16)));
 // shapes whose steady state runs in the generated loop (gen_fwd_loop.py)
 template <typename E, int D, int NW, int NS>
 constexpr bool fwd_has_generated_loop() {
-    return Elem<E>::k16 && D == 128 && NW == 8 && NS == 4;
+    return Elem<E>::k16 && ((D == 128 && NW == 8 && NS == 4) || (D == 64 && NW == 4 && NS == 3));
 }
 
 template <typename E>
@@ -374,26 +374,37 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
                 const ET* vb = vptr + (int64_t)t_issue * p.sv.t;
                 const unsigned kstep = (unsigned)(TK * p.sk.t * Elem<E>::kBytes), vstep = (unsigned)(TK * p.sv.t * Elem<E>::kBytes);
                 const unsigned w1024 = wave * 1024;
+                // Q as the loop takes it: sixteen registers per operand
                 i32x16 q0, q1;
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         q0[4 * j + e] = qf.c[j][e];
-                        q1[4 * j + e] = qf.c[4 + j][e];
+                        q1[4 * j + e] = qf.c[(NJ > 4 ? 4 : 0) + j][e];
                     }
-                if constexpr (std::is_same<E, bf16_t>::value) {
+                unsigned long long over_mask = 0;
+                const float block_hi = Lim::kBlockHi;
+                constexpr bool kBf16 = std::is_same<E, bf16_t>::value;
+                static_assert(decltype(load_k)::PER_WAVE == 3 && decltype(load_v)::PER_WAVE == 3, "three loads per wave and tile");
+                if constexpr (D == 128 && kBf16) {
                     CHILL_FWD_LOOP_BF16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, q0, q1, mneg, k_lane,
                                                 v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
                                                 load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave);
-                } else {
-                    unsigned long long over_mask = 0;
-                    const float block_hi = Lim::kBlockHi;
+                } else if constexpr (D == 128) {
                     CHILL_FWD_LOOP_F16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, over_mask, q0, q1, mneg,
                                                k_lane, v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
                                                load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
-                    over |= ((over_mask >> lane) & 1) != 0;
+                } else if constexpr (kBf16) {
+                    CHILL_FWD_LOOP_BF16_64_4_3(o[0], o[1], l_run, cnt, rem, cur, kb, vb, q0, mneg, k_lane, v_lane,
+                                               load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0], load_v.goff[1],
+                                               load_v.goff[2], lds_base, kstep, vstep, w1024, wave);
+                } else {
+                    CHILL_FWD_LOOP_F16_64_4_3(o[0], o[1], l_run, cnt, rem, cur, kb, vb, over_mask, q0, mneg, k_lane, v_lane,
+                                              load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0], load_v.goff[1],
+                                              load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
                 }
+                if (Lim::kBlockLimit) over |= ((over_mask >> lane) & 1) != 0;
                 CHILL_STAMP(4);
 #ifdef CHILL_FWD_TIMING
                 stamps[1] = (unsigned)__builtin_amdgcn_s_memtime() - clk0;  // shader clocks spent in the loop

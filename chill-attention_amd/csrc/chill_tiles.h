@@ -76,8 +76,11 @@ constexpr int kDqShortSequence = 4096;
 // The same shape is taken when the 8-wave one would leave CUs without a workgroup (B1 H8 T8192 causal:
 // forward -7 %, dQ -17 %; with twice as many heads the 8-wave shape wins again).
 constexpr int kComputeUnits = 256;
+// (forward: only dQ still takes it; the 8-wave forward with its generated loop is 23 % faster than the 4-wave
+// one at B1 H8 T8192)
 constexpr bool fwd_takes_short_row(long long batch_heads, int T) {
-    return T <= kFwdShortSequence || batch_heads * ((T + 255) / 256) <= kComputeUnits;
+    (void)batch_heads;
+    return T <= kFwdShortSequence;
 }
 constexpr bool dq_takes_short_row(long long batch_heads, int T) {
     return T <= kDqShortSequence || batch_heads * ((T + 255) / 256) <= kComputeUnits;
@@ -105,7 +108,9 @@ constexpr int fwd_stages(int mask_id, int D, int dtype, int T) {
     const int streamed = fwd_streamed(mask_id, D, dtype, T);
     if (dtype != CHILL_F32 && D <= 128) {
         if (CHILL_TUNE_FWD_STAGES) return CHILL_TUNE_FWD_STAGES;
-        if (fwd_waves(mask_id, D, dtype, T) == 4) return 2;
+        // the fast forward keeps one tile resident ahead of the one in use: three stages (two workgroups of
+        // four waves still share a CU at head dim 64), four for the 8-wave workgroup that owns its CU
+        if (fwd_waves(mask_id, D, dtype, T) == 4) return (CHILL_FWD_FAST && D == 64) ? 3 : 2;
         if (CHILL_FWD_FAST) return 4;
     }
     return 3 * fwd_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;

@@ -580,7 +580,8 @@ def main():
     ab = [x for x in args.ablate.split(",") if x]
     global ABLATE_WAITS
     ABLATE_WAITS = any(x in ab for x in ("lds", "kread", "vread", "vb128"))
-    configs = [Config("bf16", 128, 8, 4, ab), Config("f16", 128, 8, 4, ab)]
+    configs = [Config("bf16", 128, 8, 4, ab), Config("f16", 128, 8, 4, ab),
+               Config("bf16", 64, 4, 3, ab), Config("f16", 64, 4, 3, ab)]
     with open(args.output, "w") as out:
         out.write("// Generated by gen_fwd_loop.py; do not edit.\n#pragma once\n\n")
         for c in configs:

@@ -124,9 +124,12 @@ def test_tile_table():
         assert c["waves"] == waves, (p, D, c)
         if waves == 4:
             assert c["streamed"] == 64 and 2 * c["lds_bytes"] <= 160 * 1024
+    # the fast forward (16-bit, head dim 64 / 128) keeps a tile resident ahead: three stages at D = 64, four at D = 128
+    assert tile_config(causal, 64, torch.bfloat16, _lib.PASS_FWD)["lds_bytes"] == 3 * 64 * (144 + 192)
+    assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_FWD)["lds_bytes"] == 4 * 64 * (272 + 320)
     # short sequences and small grids at head dim 128: the 4-wave shape in forward (T <= 1024) and dQ (T <= 4096)
     for p, T, bh, waves in ((_lib.PASS_FWD, 1024, 128, 4), (_lib.PASS_FWD, 1025, 128, 8), (_lib.PASS_DQ, 4096, 128, 4),
-                            (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_FWD, 8192, 8, 4), (_lib.PASS_FWD, 8192, 16, 8),
+                            (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_FWD, 8192, 8, 8), (_lib.PASS_FWD, 8192, 16, 8),
                             (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 2048, 8, 4), (_lib.PASS_DKDV, 2048, 16, 8)):
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
