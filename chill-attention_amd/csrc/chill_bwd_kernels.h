@@ -808,26 +808,39 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV (wide rows)
-// Variant for rows too long for the paired kernel's LDS budget (more than 256 bytes per row):
-// Resident: 32 key rows per wave (K, V as B operands).  Streamed through the LDS ring: Q and dO
-// tiles of TQS query rows with their LSE2 / delta, for every query head of the GQA group in turn
-// (chill_bwd_dkdv.py:156).  Steps of 32 queries; S and dP of step t+1 are issued before the vector
-// work of step t.
-template <typename E, int D, int MASK, int NW, int TQS, int NS>
-__global__ __launch_bounds__(NW * 64) void dkdv_wide_kernel(BwdParams p, int n_k_tiles, int total_items,
-                                                       int wave_has_full_blocks) {
+// Variant for rows too long for the paired kernel's LDS budget (more than 256 bytes per row: fp32 at
+// head dims 128 and 256).  A 32-key block keeps 32 x D of K, 32 x D of V and two 32 x D accumulators:
+// four times D registers per lane in one wave, more than a wave has from D = 128 on.  So SPLIT waves
+// share a block and each holds a quarter of that state per pair of waves:
+//   * wave g of the block computes a PARTIAL product over its share of the head dim, S = Q K^T for
+//     even g and dP = dO V^T for odd g, from its resident slice of K or V (B operands);
+//   * the partial products meet in LDS; behind a barrier every wave of the block adds them up and
+//     computes P and dS for itself (vector work that is small next to fp32 MFMAs);
+//   * wave g accumulates the head-dim blocks [g * DB / SPLIT, (g + 1) * DB / SPLIT) of dV^T += dO^T P
+//     and dK^T += Q^T dS.
+// Every wave issues the same number of MFMAs and none is issued twice.  Streamed through the LDS ring:
+// Q and dO tiles of 32 query rows, for every query head of the GQA group in turn
+// (chill_bwd_dkdv.py:156), with the LSE2 / delta of those rows.
+template <typename E, int D, int MASK, int NW, int SPLIT, int NS>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(D >= 256 ? 1 : 2))) void dkdv_split_kernel(BwdParams p, int n_k_tiles, int total_items,
+                                                        int wave_has_full_blocks) {
     using ET = typename Elem<E>::type;
-    constexpr int TKR = NW * 32;  // resident key rows per workgroup
+    typedef LdsTile<E, D> L;
+    static_assert(!Elem<E>::k16, "fp32 rows (16-bit rows of this length have a kernel of their own)");
+    constexpr int TQS = 32;
+    constexpr int NKB = NW / SPLIT;   // 32-key blocks per workgroup
+    constexpr int TKR = NKB * 32;     // key rows per workgroup
     constexpr int NT = NW * 64;
-    constexpr int QB = TQS / 32;
-    constexpr int DB = (D + 31) / 32;
-    constexpr int NJ = Resident<E, D>::NJ;
-    constexpr int TILE_BYTES = LdsTile<E, D>::bytes(TQS);
+    constexpr int DB = D / 32;
+    constexpr int DBW = DB / SPLIT;   // head-dim blocks a wave accumulates
+    constexpr int PARTS = SPLIT / 2;  // slices of the head dim in the partial products
+    constexpr int NJW = (L::CH / 2) / PARTS;  // 16-byte chunk pairs of a slice
+    constexpr int TILE_BYTES = L::bytes(TQS);
     constexpr int VEC_BYTES = TQS * 4;
     constexpr int STAGE_BYTES = 2 * TILE_BYTES + 2 * VEC_BYTES;  // Q, dO, LSE2, delta
-    constexpr int LA = NS - 2;
-    static_assert(NS == 2 || NS == 3, "two or three LDS stages");
-    static_assert(TQS <= 64, "one wave instruction stages a vector");
+    constexpr int X_BYTES = 16 * 64 * 4;                         // one partial product
+    static_assert(NS == 2, "two ring stages");
+    static_assert(SPLIT % 2 == 0 && DB % SPLIT == 0 && NW % SPLIT == 0, "whole shares");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int item = xcd_contiguous_item(blockIdx.x, total_items);
@@ -841,6 +854,10 @@ __global__ __launch_bounds__(NW * 64) void dkdv_wide_kernel(BwdParams p, int n_k
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kblk = wave % NKB;
+    const int g = wave / NKB;       // place among the waves of the block
+    const int role = g & 1;         // 0: S from K, 1: dP from V
+    const int part = g >> 1;        // slice of the head dim in the partial product
     const int n = lane & 31;
     const int h = lane >> 5;
 
@@ -864,11 +881,11 @@ __global__ __launch_bounds__(NW * 64) void dkdv_wide_kernel(BwdParams p, int n_k
     AsyncSwizzledLoader<E, D, TQS, NT> load_q, load_do;
     load_q.init(p.sq.t, wave, lane);
     load_do.init(p.sdo.t, wave, lane);
-    // iteration it = (group head g, q-tile): stage it % NS
+    // iteration it = (group head, q-tile): stage it % 2
     auto issue_iter = [&](int it, int st_index) {
-        const int g = it / n_tiles;
+        const int gh = it / n_tiles;
         const int q0 = (wg.start + it % n_tiles) * TQS;
-        const int hq = hkv * p.group + g;
+        const int hq = hkv * p.group + gh;
         char* st = smem + st_index * STAGE_BYTES;
         const ET* qptr = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h;
         const ET* doptr = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h;
@@ -890,116 +907,171 @@ __global__ __launch_bounds__(NW * 64) void dkdv_wide_kernel(BwdParams p, int n_k
             }
         }
     };
-#pragma unroll
-    for (int i = 0; i <= LA; i++)
-        if (i < n_iters) issue_iter(i, i);
+    if (n_iters > 0) issue_iter(0, 0);
 
-    const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
-    const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
-    const int kw = kb0 + 32 * wave;
+    // this wave's slice of K (role 0) or V (role 1): chunk pairs [part * NJW, (part + 1) * NJW) of the
+    // block's 32 rows as B operands; rows past the end of the tensor read as zero
+    const int kw = kb0 + 32 * kblk;
     const int k_pos = kw + n;
-    OperandOffsets<E, D> ofs;
-    ofs.init(lane);
-    Resident<E, D> kf, vf;
-    load_resident<E, D>(kf, kptr + (int64_t)kw * p.sk.t, p.sk.t, p.T - kw, lane);
-    load_resident<E, D>(vf, vptr + (int64_t)kw * p.sv.t, p.sv.t, p.T - kw, lane);
+    i32x4 res[NJW];
+    {
+        const ET* src = role == 0 ? reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h
+                                  : reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
+        const int64_t stride = role == 0 ? p.sk.t : p.sv.t;
+#pragma unroll
+        for (int j = 0; j < NJW; j++) {
+            i32x4 val = {0, 0, 0, 0};
+            if (k_pos < p.T)
+                val = *reinterpret_cast<const i32x4*>(reinterpret_cast<const char*>(src + (int64_t)k_pos * stride) +
+                                                      (2 * (part * NJW + j) + h) * 16);
+            res[j] = val;
+        }
+    }
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
     if (kw < seq_len) wr = tile_range<MASK, false>(kw, 32, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
     const int ta = wr.start - wg.start, tb = wr.end - wg.start;
     const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
 
-    f32x16 dk[DB], dv[DB];
+    f32x16 dk[DBW], dv[DBW];
 #pragma unroll
-    for (int i = 0; i < DB; i++)
+    for (int i = 0; i < DBW; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             dk[i][r] = 0.f;
             dv[i][r] = 0.f;
         }
     const float scale = p.scale_log2;
-
-    // S = Q K^T and dP = dO V^T of step qb of the stage at `stage`
-    auto gemms = [&](f32x16& sdst, f32x16& dpdst, const lds_char* stage, int qb) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            sdst[r] = 0.f;
-            dpdst[r] = 0.f;
-        }
-        sdst = mma_rowwise<E, D>(stage, qb, ofs, kf, sdst, lane);
-        dpdst = mma_rowwise<E, D>(stage + TILE_BYTES, qb, ofs, vf, dpdst, lane);
-    };
-
-    f32x16 s[2], dp[2];
     const lds_char* lds0 = (const lds_char*)smem;
-#pragma unroll
-    for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(kf.c[j]), "v"(vf.c[j]));
+    // the partial products of block kblk: SPLIT slots of 16 x 64 floats, register r of lane l at
+    // ((r / 4) * 64 + l) * 16 + (r % 4) * 4
+    char* xblock = smem + 2 * STAGE_BYTES + kblk * SPLIT * X_BYTES;
+    // this wave's head-dim blocks in the accumulation: columns 32 * (g * DBW + i) + n of the Q / dO tiles
+    const int db0 = g * DBW;
 
-    int st_cur = NS - 1;
-    int st_issue = LA;
     int tile = -1;  // position of iteration `it` inside the q-tile range (it % n_tiles)
-    bool have_cur = false;  // s[0] / dp[0] already hold the first step of this iteration
     for (int it = 0; it < n_iters; it++) {
         wait_async_tiles();
-        __syncthreads();
-        st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
-        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        __syncthreads();  // tile `it` is in LDS; every wave is done with the iteration before
         tile = tile + 1 == n_tiles ? 0 : tile + 1;
-        if (it + LA + 1 < n_iters) issue_iter(it + LA + 1, st_issue);
-        if (tile < ta || tile >= tb) {
-            have_cur = false;
-            continue;
-        }
-        const lds_char* stage = lds0 + st_cur * STAGE_BYTES;
-        const lds_char* stage_next = lds0 + (st_cur + 1 == NS ? 0 : st_cur + 1) * STAGE_BYTES;
-        const lds_float* vec = reinterpret_cast<const lds_float*>(stage + 2 * TILE_BYTES);
-        const bool full = (tile >= fa) && (tile < fb);
+        const bool mine = tile >= ta && tile < tb;  // (the same for all waves of a block)
+        const lds_char* stage = lds0 + (it & 1) * STAGE_BYTES;
         const int q0 = (wg.start + tile) * TQS;
-        // the next iteration is one of mine if it is the next tile of my range, or the first tile
-        // of my range for the next head of the group
-        const int tile_next = tile + 1 == n_tiles ? 0 : tile + 1;
-        const bool next_mine = (it + 1 < n_iters) && tile_next >= ta && tile_next < tb;
-        if (!have_cur) gemms(s[0], dp[0], stage, 0);
-
+        // The wave that produces S (dP) also subtracts the LSE2 (delta) of its query rows, rows
+        // 8 * (r / 4) + 4 * h + r % 4 of the tile: every wave reads one of the two vectors and only where
+        // it produces.
+        if (it + 1 < n_iters) issue_iter(it + 1, (it + 1) & 1);
+        // LDS offsets are derived from these inside the iteration: kept across iterations they would
+        // take more registers than the few vector instructions that compute them save
+        int n_it = n, h_it = h;
+        asm volatile("" : "+v"(n_it), "+v"(h_it));
+        if (mine) {
+            const lds_char* src = stage + role * TILE_BYTES;
+            f32x16 part_acc;
 #pragma unroll
-        for (int qb = 0; qb < QB; qb++) {
-            f32x16& cs = s[qb & 1];
-            f32x16& cdp = dp[qb & 1];
-            if (qb + 1 < QB) {
-                gemms(s[(qb + 1) & 1], dp[(qb + 1) & 1], stage, qb + 1);
-            } else if (LA >= 1 && next_mine) {
-                gemms(s[(qb + 1) & 1], dp[(qb + 1) & 1], stage_next, 0);
+            for (int r = 0; r < 16; r++) part_acc[r] = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJW; j++) {
+                const i32x4 a = *reinterpret_cast<const lds_i32x4*>(src + L::chunk_off(n_it, 2 * (part * NJW + j) + h_it));
+                part_acc = Elem<E>::mma(a, res[j], part_acc);
             }
-            f32x4 lse4[4], del4[4];
+            float vec16[16];
+            const lds_float* vec = reinterpret_cast<const lds_float*>(stage + 2 * TILE_BYTES) + role * TQS;
 #pragma unroll
             for (int g4 = 0; g4 < 4; g4++) {
-                lse4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 32 * qb + 8 * g4 + 4 * h);
-                del4[g4] = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + TQS + 32 * qb + 8 * g4 + 4 * h);
+                const f32x4 v4 = *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>(vec + 8 * g4 + 4 * h_it);
+#pragma unroll
+                for (int e = 0; e < 4; e++) vec16[4 * g4 + e] = v4[e];
             }
-            auto pos = [&](int r, int& q, int& k, float& lse, float& delta) {
-                q = q0 + 32 * qb + 8 * (r / 4) + 4 * h + (r % 4);
-                k = k_pos;
-                lse = lse4[r / 4][r % 4];
-                delta = del4[r / 4][r % 4];
-            };
-            if (full)
-                softmax_grad_block<MASK, false>(cs, cdp, scale, seq_len, p.margs, pos);
-            else
-                softmax_grad_block<MASK, true>(cs, cdp, scale, seq_len, p.margs, pos);
-            mma_transposed<E, D>(stage + TILE_BYTES, qb, ofs, cs, dv, lane);  // dV^T += dO^T P
-            mma_transposed<E, D>(stage, qb, ofs, cdp, dk, lane);              // dK^T += Q^T dS
+            // s * scale - LSE2 (what the exponential takes, chill_bwd_dkdv.py:378) or dP - delta
+            const float mult = role == 0 ? scale : 1.f;
+            const bool sub = part == 0;
+#pragma unroll
+            for (int r = 0; r < 16; r++) part_acc[r] = part_acc[r] * mult - (sub ? vec16[r] : 0.f);
+            f32x4* out = reinterpret_cast<f32x4*>(xblock + g * X_BYTES);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++)
+                out[r4 * 64 + lane] = f32x4{part_acc[4 * r4], part_acc[4 * r4 + 1], part_acc[4 * r4 + 2], part_acc[4 * r4 + 3]};
         }
-        have_cur = LA >= 1 && next_mine;
-        if ((QB & 1) && have_cur) {
-            s[0] = s[1];
-            dp[0] = dp[1];
+        // the first operands of the accumulation do not depend on the exchange
+        float a_do[2][DBW], a_q[2][DBW];
+        auto read_operands = [&](int r, int buf) {
+            const int rw = 8 * (r / 4) + 4 * h_it + (r % 4);
+#pragma unroll
+            for (int i = 0; i < DBW; i++) {
+                const int off = L::elem_off(rw, 32 * (db0 + i) + n_it);
+                a_do[buf][i] = *reinterpret_cast<const lds_float*>(stage + TILE_BYTES + off);
+                a_q[buf][i] = *reinterpret_cast<const lds_float*>(stage + off);
+            }
+        };
+        if (mine) read_operands(0, 0);
+        __syncthreads();  // the partial products of this iteration are in LDS
+        if (!mine) continue;
+
+        f32x16 cs, cdp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            cs[r] = 0.f;
+            cdp[r] = 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < PARTS; e++) {
+            const f32x4* xs = reinterpret_cast<const f32x4*>(xblock + (2 * e) * X_BYTES);
+            const f32x4* xd = reinterpret_cast<const f32x4*>(xblock + (2 * e + 1) * X_BYTES);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const f32x4 a = xs[r4 * 64 + lane], d = xd[r4 * 64 + lane];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    cs[4 * r4 + i] += a[i];
+                    cdp[4 * r4 + i] += d[i];
+                }
+            }
+        }
+        const bool full = (tile >= fa) && (tile < fb);
+        // P = exp2(s * scale - LSE2) and dS = P (dP - delta) (the sums hold the arguments), then
+        // dV^T += dO^T P and dK^T += Q^T dS over this wave's head-dim blocks: the contraction runs over the
+        // 32 query rows, two per MFMA (rows 8 * (r / 4) + r % 4 and that + 4).  Register by register, so
+        // that the vector work and the LDS reads of one register run under the MFMAs of the one before.
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float pv = fast_exp2(cs[r]);
+            if (!full) {
+                const int qq = q0 + 8 * (r / 4) + 4 * h + (r % 4);
+                const bool ok = (qq < seq_len) && (k_pos < seq_len) && Mask<MASK>::pred(qq, k_pos, seq_len, p.margs);
+                pv = ok ? pv : 0.f;
+            }
+            const float ds = pv * cdp[r];
+            if (r + 1 < 16) read_operands(r + 1, (r + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < DBW; i++) {
+                dv[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_do[r & 1][i], pv, dv[i], 0, 0, 0);
+                dk[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_q[r & 1][i], ds, dk[i], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 
+    // lane (n, h) holds columns d = 32 * (db0 + i) + 8 * (r / 4) + 4 * h + r % 4 of ITS key row
     if (k_pos < p.T) {
         const bool valid = k_pos < seq_len;
-        store_row_transposed<E, D>(dkbase + (int64_t)k_pos * p.sdk.t, dk, p.sm_scale, valid, h);
-        store_row_transposed<E, D>(dvbase + (int64_t)k_pos * p.sdv.t, dv, 1.f, valid, h);
+        float* dkrow = reinterpret_cast<float*>(dkbase + (int64_t)k_pos * p.sdk.t);
+        float* dvrow = reinterpret_cast<float*>(dvbase + (int64_t)k_pos * p.sdv.t);
+#pragma unroll
+        for (int i = 0; i < DBW; i++)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                const int d0 = 32 * (db0 + i) + 8 * g4 + 4 * h;
+                f32x4 a, c;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    a[e] = valid ? dk[i][4 * g4 + e] * p.sm_scale : 0.f;
+                    c[e] = valid ? dv[i][4 * g4 + e] : 0.f;
+                }
+                *reinterpret_cast<f32x4*>(dkrow + d0) = a;
+                *reinterpret_cast<f32x4*>(dvrow + d0) = c;
+            }
     }
 }
 
@@ -1010,7 +1082,8 @@ int launch_dkdv_shape(const BwdParams& p, hipStream_t stream) {
     constexpr int CB = dkdv_regs_blocks(D, Elem<E>::kDType);
     constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType) && CB == 0;
     static_assert(CB > 0 ? (cfg.rows == 128 * CB && cfg.streamed == 32 && cfg.waves == 4)
-                         : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64) : (cfg.rows == cfg.waves * 32),
+                         : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64)
+                                  : (cfg.rows * dkdv_split(D) == cfg.waves * 32 && cfg.streamed == 32),
                   "tile table and kernel shape disagree");
     const int n_k_tiles = cdiv(p.T, cfg.rows);
     const int64_t total64 = (int64_t)p.B * p.H_kv * n_k_tiles;
@@ -1024,7 +1097,7 @@ int launch_dkdv_shape(const BwdParams& p, hipStream_t stream) {
     else if constexpr (paired)
         kern = dkdv_kernel<E, D, MASK_ID, cfg.waves, 2>;
     else
-        kern = dkdv_wide_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, dkdv_wide_stages(cfg.streamed, D, Elem<E>::kDType)>;
+        kern = dkdv_split_kernel<E, D, MASK_ID, cfg.waves, dkdv_split(D), 2>;
     // mask rule order is (q tile, k tile): the streamed tile is the q tile here
     const bool hfb = Mask<MASK_ID>::has_full_blocks(cfg.streamed, CB > 0 ? 32 * CB : 32, p.T, p.margs);
     if (cfg.lds_bytes > 48 * 1024) {

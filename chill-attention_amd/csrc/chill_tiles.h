@@ -161,8 +161,7 @@ constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype, int T = kLong
 // dK/dV, rows of at most 256 bytes ("paired" kernel): a workgroup of 8 waves owns 128 key rows;
 // pairs of waves share a 32-key block and split the streamed 64-row query tiles.  LDS: the resident
 // K and V tiles plus two ring stages of swizzled Q and dO tiles with the LSE2 and delta of their rows.
-// Longer rows ("wide" kernel): 4 waves own 128 key rows with K, V resident in registers; the ring
-// holds 32-row Q and dO tiles.
+// Longer rows: dkdv_split_kernel, below.
 constexpr bool dkdv_is_paired(int D, int dtype) { return D * elem_bytes(dtype) <= 256; }
 // 16-bit head dims <= 64: workgroups of 4 waves (64 key rows), small enough in LDS (50 KiB at D = 64)
 // and registers (167) for two or three of them per CU, which hide each other's start and end
@@ -182,11 +181,15 @@ constexpr bool dkdv_takes_small_row(long long batch_kv_heads, int T) {
 // at the end the waves of a pair exchange one fp32 accumulator each through LDS: 8 waves x (D rounded
 // up to 32) x 32 floats
 constexpr int dkdv_paired_exchange_bytes(int D) { return 8 * ((D + 31) / 32) * 16 * 64 * 4; }
-constexpr int dkdv_wide_stage_bytes(int streamed, int D, int dtype) {
-    return 2 * streamed * D * elem_bytes(dtype) + 2 * streamed * 4;
-}
-constexpr int dkdv_wide_stages(int streamed, int D, int dtype) {
-    return 3 * dkdv_wide_stage_bytes(streamed, D, dtype) <= 144 * 1024 ? 3 : 2;
+// Longer rows (fp32 at head dims 128 and 256, dkdv_split_kernel): dkdv_split(D) waves share a 32-key
+// block and its state; two ring stages of 32-row Q and dO tiles, then one 4 KiB slot per wave for the
+// partial products.  Head dim 128: 8 waves, 128 key rows, two waves per SIMD; head dim 256: 4 waves
+// on one 32-key block (two ring stages alone take 128 KiB).
+constexpr int dkdv_split(int D) { return D >= 256 ? 4 : 2; }
+constexpr int dkdv_split_waves(int D) { return D >= 256 ? 4 : 8; }
+constexpr int dkdv_split_stage_bytes(int D, int dtype) { return 2 * 32 * D * elem_bytes(dtype) + 2 * 32 * 4; }
+constexpr int dkdv_split_lds_bytes(int D, int dtype) {
+    return 2 * dkdv_split_stage_bytes(D, dtype) + dkdv_split_waves(D) * 16 * 64 * 4;
 }
 
 // dK/dV with hand-managed accumulation registers (dkdv_regs_kernel, 16-bit inputs): 4 waves, K in
@@ -216,7 +219,7 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype, bool small_
         const int exchange = dkdv_paired_exchange_bytes(D) * waves / 8;
         return TileConfig{rows, 64, waves, ring > exchange ? ring : exchange};
     }
-    return TileConfig{128, 32, 4, dkdv_wide_stages(32, D, dtype) * dkdv_wide_stage_bytes(32, D, dtype)};
+    return TileConfig{32 * dkdv_split_waves(D) / dkdv_split(D), 32, dkdv_split_waves(D), dkdv_split_lds_bytes(D, dtype)};
 }
 
 // batch_heads = B * H and T = sequence length of the launch (the forward and dQ rows depend on them);

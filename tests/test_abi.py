@@ -108,9 +108,13 @@ def test_tile_table():
             for D in (16, 32, 64, 128, 256):
                 for p in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKDV):
                     c = tile_config(mask, D, dt, p)
-                    # one wave per 32 resident rows, or (dK/dV) a pair of waves per 32 rows
-                    assert c["rows"] in (32 * c["waves"], 16 * c["waves"]) and c["streamed"] % 32 == 0
+                    # one wave per 32 resident rows, or (dK/dV) two or four waves per 32 rows
+                    assert c["rows"] in (32 * c["waves"], 16 * c["waves"], 8 * c["waves"]) and c["streamed"] % 32 == 0
                     assert 0 < c["lds_bytes"] <= 160 * 1024
+    # fp32 rows of 512 bytes and more: the waves of a 32-key block split its state
+    assert tile_config(ca.CausalChillMask(), 128, torch.float32, _lib.PASS_DKDV)["waves"] == 8
+    assert tile_config(ca.CausalChillMask(), 128, torch.float32, _lib.PASS_DKDV)["rows"] == 128
+    assert tile_config(ca.CausalChillMask(), 256, torch.float32, _lib.PASS_DKDV)["rows"] == 32
     # rows the tile sweep put into the table (mask- and head-dim-specific)
     causal, window = ca.CausalChillMask(), ca.SlidingWindowChillMask(128, 128)
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 64
