@@ -99,6 +99,39 @@ EXPORTED_SYMBOLS = (
 
 BWD_NOALLOC_MAX_ROWS = 4 * 1024 * 1024  # CHILL_BWD_NOALLOC_MAX_ROWS of the header
 
+# The eager-mode operator registered from C++ (csrc/chill_torch.cpp): the same adapters and autograd
+# formula as the torch.library layer of chill.py without its per-call Python cost.  It links against no
+# kernel library; a call names the entry points it is to use through a table built here.
+TORCH_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libchill_attention_torch.so")
+
+
+class EntryPoints(ctypes.Structure):
+    """Addresses of one kernel library's entry points, in the order csrc/chill_torch.cpp declares."""
+
+    _fields_ = [(n, c_void_p) for n in ("fwd", "delta", "dkdv", "dq", "status_string")]
+
+
+def entry_points(cdll: ctypes.CDLL) -> EntryPoints:
+    names = ("chill_fwd", "chill_bwd_delta", "chill_bwd_dkdv", "chill_bwd_dq", "chill_status_string")
+    return EntryPoints(*(ctypes.cast(getattr(cdll, n), c_void_p).value for n in names))
+
+
+_torch_operator = False  # not looked for yet
+
+
+def torch_operator():
+    """``torch.ops.chill_attention_amd.attention``, or None when its library has not been built or
+    CHILL_ATTENTION_EAGER_OP=0 asks for the Python operator layer."""
+    global _torch_operator
+    if _torch_operator is False:
+        _torch_operator = None
+        if os.environ.get("CHILL_ATTENTION_EAGER_OP", "1") != "0" and os.path.exists(TORCH_LIB_PATH):
+            import torch
+
+            torch.ops.load_library(TORCH_LIB_PATH)
+            _torch_operator = torch.ops.chill_attention_amd.attention
+    return _torch_operator
+
 
 def check(fn: str, status: int) -> int:
     """Raise for a negative status, pass non-negative values through."""

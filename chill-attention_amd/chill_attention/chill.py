@@ -271,6 +271,23 @@ def _chill_reference_naive(
     return out * res_mask, res_mask
 
 
+# mask class -> (C++ operator or None, entry-point table of the class's kernel library, mask id)
+_eager = {}
+
+
+def _eager_operator(mask: ChillMask):
+    cls = type(mask)
+    entry = _eager.get(cls)
+    if entry is None:
+        op = _lib.torch_operator()
+        table = mask_id = None
+        if op is not None:
+            table = _lib.entry_points(cls._library())
+            mask_id = _descriptor(cls, mask.constargs).id
+        entry = _eager[cls] = (op, table, mask_id)
+    return entry
+
+
 def _chill_attention(q, k, v, lens, mask_name, mask_args, sm_scale, return_lse, prescale_qk, precision, autotune):
     requires_grad = any(i.requires_grad for i in (q, k, v))
     forward = getattr(torch.ops.chill_attention, f"forward{mask_name}")
@@ -311,12 +328,22 @@ def chill_attention(
         ``O`` or ``(O, LSE2)``.
     """
     register_chill_mask(mask)
+    if sm_scale is None:
+        sm_scale = 1.0 / (q.shape[-1] ** 0.5)
+    if not torch.compiler.is_compiling():
+        # eager calls take the operator registered from C++ (same adapters, same autograd formula);
+        # the torch.library operators below serve torch.compile and builds without that library
+        op, table, mask_id = _eager_operator(mask)
+        if op is not None:
+            _check_inputs(q, k, v, lens, sm_scale)
+            mask_args = [int(a) for a in mask.constargs]
+            _require(all(a == b for a, b in zip(mask_args, mask.constargs)), "mask arguments must be integers")
+            O, LSE = op(q, k, v, lens, ctypes.addressof(table), mask_id, mask_args, float(sm_scale), bool(return_lse))
+            return (O, LSE) if return_lse else O
     if not torch.compiler.is_compiling():
         for i in (q, k, v):
             torch._dynamo.mark_static(i, 1)
             torch._dynamo.mark_static(i, 3)
-    if sm_scale is None:
-        sm_scale = 1.0 / (q.shape[-1] ** 0.5)
     return _chill_attention(
         q=q, k=k, v=v, lens=lens, mask_name=mask.name, mask_args=mask.constargs, sm_scale=sm_scale,
         return_lse=return_lse, prescale_qk=prescale_qk, precision=precision, autotune=autotune,
