@@ -405,6 +405,7 @@ __device__ __forceinline__ void fwd_q_tile(const FwdParams& p, char* smem, int b
 }  // namespace chill
 #include "chill_fwd_regs.h"
 #include "chill_fwd_fast.h"
+#include "chill_fwd_small.h"
 namespace chill {
 
 // Shapes served by fwd_q_tile_fast (16-bit inputs, head dim 64 or 128, 64-key tiles with one resident
@@ -494,6 +495,23 @@ int launch_fwd_shape(const FwdParams& p, hipStream_t stream) {
     return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
 }
 
+// A launch far too small for the chip: 32 query rows per workgroup, the keys split over its waves.
+template <typename E, int D, int MASK_ID>
+int launch_fwd_small(const FwdParams& p, hipStream_t stream) {
+    constexpr int kLdsBytes = fwd_small_lds_bytes(D, Elem<E>::kDType);
+    const int n_q_tiles = cdiv(p.T, 32);
+    const int total = p.B * p.H * n_q_tiles;  // (at most kComputeUnits / 4 * 4 * 32 by fwd_takes_small)
+    void (*kern)(FwdParams, int, int, int) = fwd_small_kernel<E, D, MASK_ID>;
+    const bool hfb = Mask<MASK_ID>::has_full_blocks(32, 32, p.T, p.margs);
+    if (kLdsBytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsBytes) != hipSuccess)
+            return CHILL_ERR_HIP;
+    }
+    hipLaunchKernelGGL(kern, dim3(total), dim3(kFwdSmallWaves * 64), kLdsBytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
+    return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+}
+
 template <typename E, int D>
 int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
     // the async loader keeps per-lane global offsets in 32 bits
@@ -504,7 +522,11 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         // the table has a row of its own for short sequences and small grids where that row differs
         constexpr bool has_short_row = fwd_tile_config(MASK_ID, D, Elem<E>::kDType, 1).waves !=
                                        fwd_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
-        if constexpr (has_short_row) {
+        bool small = false;
+        if constexpr (D * Elem<E>::kBytes <= 512) small = fwd_takes_small((long long)p.B * p.H, p.T, D, Elem<E>::kDType);
+        if (small) {
+            if constexpr (D * Elem<E>::kBytes <= 512) status = launch_fwd_small<E, D, MASK_ID>(p, stream);
+        } else if constexpr (has_short_row) {
             status = fwd_takes_short_row((long long)p.B * p.H, p.T) ? launch_fwd_shape<E, D, MASK_ID, true>(p, stream)
                                                                     : launch_fwd_shape<E, D, MASK_ID, false>(p, stream);
         } else {

@@ -118,6 +118,21 @@ constexpr int fwd_stages(int mask_id, int D, int dtype, int T) {
 // 16-bit inputs at head dim 256: fwd_regs_kernel (O^T in hand-managed accumulation registers).
 constexpr bool fwd_uses_regs(int D, int dtype) { return dtype != CHILL_F32 && D == 256; }
 
+// Forward launches far too small for the chip (fwd_small_kernel): a workgroup of four waves owns 32
+// query rows and its waves split the keys.  Per wave LDS holds a 32-row K block, a 32-row V block and
+// the wave's running max and row sum; rows of at most 512 bytes, so that four such areas fit.
+constexpr int kFwdSmallWaves = 4;
+constexpr int kFwdSmallMaxT = 1024;
+// (at the end the area also takes the wave's partial O^T, 4 KiB per 32 columns of the head dim)
+constexpr int fwd_small_wave_bytes(int D, int dtype) {
+    const int blocks = 2 * 32 * D * elem_bytes(dtype), partial = ((D + 31) / 32) * 16 * 64 * 4;
+    return (blocks > partial ? blocks : partial) + 2 * 64 * 4;
+}
+constexpr int fwd_small_lds_bytes(int D, int dtype) { return kFwdSmallWaves * fwd_small_wave_bytes(D, dtype); }
+constexpr bool fwd_takes_small(long long batch_heads, int T, int D, int dtype) {
+    return D * elem_bytes(dtype) <= 512 && T <= kFwdSmallMaxT && batch_heads * ((T + 127) / 128) <= kComputeUnits / 4;
+}
+
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {
     const int waves = fwd_waves(mask_id, D, dtype, T);
     const int streamed = fwd_streamed(mask_id, D, dtype, T);
@@ -229,6 +244,10 @@ inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_
     if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
     switch (pass) {
         case CHILL_PASS_FWD:
+            if (T != kLongSequence && fwd_takes_small(batch_heads, T, D, dtype)) {
+                *out = TileConfig{32, 32, kFwdSmallWaves, fwd_small_lds_bytes(D, dtype)};
+                return CHILL_OK;
+            }
             *out = fwd_tile_config(mask_id, D, dtype, (T != kLongSequence && fwd_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
             return CHILL_OK;
         case CHILL_PASS_DQ:

@@ -15,6 +15,7 @@ import pytest
 import torch
 
 import chill_attention as ca
+from chill_attention import _lib
 from conftest import MASK_INSTANCES, make_mask, mask_id
 from oracle import chill_oracle as orc
 
@@ -78,7 +79,11 @@ def make_qkv(shape, dtype, noncontiguous):
 
 
 # (noncontiguous, head_dim, B, (H, H_kv)) combinations covering every value of the reference matrix
-FWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (6, 3)), (False, 128, 1, (6, 1)), (True, 16, 7, (8, 8))]
+# Launches of at most 64 workgroups' worth of rows at T <= 1024 take the forward that splits the keys of
+# a q-tile over its waves; (11, (6, 3)) keeps the ordinary forward covered at the short lengths, the
+# shapes with B = 1 cover the other one at the longer ones.
+FWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (6, 3)), (False, 128, 1, (6, 1)), (True, 16, 7, (8, 8)),
+              (False, 64, 11, (6, 3))]
 BWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (8, 2)), (False, 128, 16, (6, 1)), (True, 16, 7, (8, 8)),
               (False, 128, 1, (8, 1))]
 
@@ -130,6 +135,64 @@ def test_backward_matrix(m, dtype, lens_kind, T):
         for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
             assert torch.isfinite(got).all(), name
             check_close(got, want, dtype, GRAD_TOL[dtype], D, f"{name} {tag}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16], ids=str)
+@pytest.mark.parametrize("m", MASK_INSTANCES, ids=mask_id)
+def test_small_launch_forward(m, dtype):
+    """The forward of launches far too small for the chip (32 query rows per workgroup, keys split over
+    its waves, partial softmax states merged at the end): every mask instance, ragged lengths, GQA,
+    rows that see no key, LSE included, against the oracle; and the same rows through the ordinary
+    forward (the same problem with enough batch entries) within rounding."""
+    mask = make_mask(m)
+    rng = np.random.default_rng(stable_seed(m, str(dtype), "small"))
+    for T, D, (H, Hkv) in ((1000, 64, (4, 2)), (333, 128, (2, 1)), (1024, 32, (3, 3)), (77, 16, (2, 2))):
+        B = 2
+        q, k, v = (make_qkv((B, h, T, D), dtype, False) for h in (H, Hkv, Hkv))
+        lens = torch.tensor([T, max(1, T // 3)], dtype=torch.int32, device=DEV)
+        ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), lens)
+        out, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens, return_lse=True)
+        check_close(out * res_mask, ref, dtype, OUT_TOL[dtype], D, f"O small launch T={T} D={D}")
+        # the ordinary forward on the same rows: 40 copies of the batch make the launch large
+        rep = 40
+        big, big_lse = ca.chill_attention(q.repeat(rep, 1, 1, 1), k.repeat(rep, 1, 1, 1), v.repeat(rep, 1, 1, 1),
+                                          mask=mask, lens=lens.repeat(rep), return_lse=True)
+        torch.testing.assert_close(out.float(), big[:B].float(), atol=OUT_TOL[dtype][0], rtol=OUT_TOL[dtype][1])
+        finite = torch.isfinite(big_lse[:B])
+        assert (torch.isfinite(lse) == finite).all()
+        # (the ordinary forward of 16-bit inputs folds the scale into Q and rounds it once more, as the
+        # reference's PRESCALE_QK does, chill_fwd.py:158-159: its scores carry that rounding)
+        lse_atol = {torch.float32: 1e-4, torch.float16: 5e-3, torch.bfloat16: 3e-2}[dtype]
+        torch.testing.assert_close(lse[finite], big_lse[:B][finite], atol=lse_atol, rtol=1e-4)
+        assert (lse[~finite] == big_lse[:B][~finite]).all()
+
+
+def test_cpp_operator_matches_python_operator():
+    """Eager calls go through the operator registered from C++; the torch.library operators (what
+    torch.compile sees) must give the same bits, forward and backward, on the same kernels."""
+    assert _lib.torch_operator() is not None, "libchill_attention_torch.so has not been built"
+    mask = ca.SlidingWindowChillMask(100, 20)
+    B, H, Hkv, T, D = 3, 4, 2, 700, 64
+    q = make_qkv((B, H, T, D), torch.bfloat16, True).requires_grad_()
+    k = make_qkv((B, Hkv, T, D), torch.bfloat16, True).requires_grad_()
+    v = make_qkv((B, Hkv, T, D), torch.bfloat16, False).requires_grad_()
+    lens = torch.tensor([T, 1, 333], dtype=torch.int32, device=DEV)
+    do = make_qkv((B, H, T, D), torch.bfloat16, False)
+    out, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens, return_lse=True)
+    out.backward(do)
+    got = [out.detach(), lse.detach()] + [x.grad.clone() for x in (q, k, v)]
+    for x in (q, k, v):
+        x.grad = None
+    from chill_attention import chill as chill_mod
+
+    out2, lse2 = chill_mod._chill_attention(q, k, v, lens, mask.name, mask.constargs, D ** -0.5, True, False, "ieee", False)
+    out2.backward(do)
+    want = [out2.detach(), lse2.detach()] + [x.grad for x in (q, k, v)]
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    # no gradient asked for: no LSE is kept, the output is the same
+    with torch.no_grad():
+        assert torch.equal(ca.chill_attention(q, k, v, mask=mask, lens=lens), out2.detach())
 
 
 @pytest.mark.parametrize("D", [32, 64, 256])
