@@ -18,6 +18,9 @@
 #ifndef CHILL_TUNE_FWD_STREAMED
 #define CHILL_TUNE_FWD_STREAMED 0
 #endif
+#ifndef CHILL_TUNE_FWD_SMALL
+#define CHILL_TUNE_FWD_SMALL 1
+#endif
 #ifndef CHILL_TUNE_FWD_STAGES
 #define CHILL_TUNE_FWD_STAGES 0
 #endif
@@ -121,8 +124,13 @@ constexpr bool fwd_uses_regs(int D, int dtype) { return dtype != CHILL_F32 && D 
 // Forward launches far too small for the chip (fwd_small_kernel): a workgroup of four waves owns 32
 // query rows and its waves split the keys.  Per wave LDS holds a 32-row K block, a 32-row V block and
 // the wave's running max and row sum; rows of at most 512 bytes, so that four such areas fit.
+// It is taken while its grid of B * H * T / 32 workgroups is about what the chip holds at once
+// (measured against the ordinary forward, causal and full masks, T = 128 .. 4096, 1 .. 128 heads: with
+// up to 256 workgroups it wins everywhere, by 1.1x .. 1.5x for 16-bit inputs and up to 3.6x for fp32; with
+// 512 it still wins for fp32 and at head dim 128, where a block is more work, and loses 10-20 % at
+// head dim 64 and below; with 1024 it loses or ties).
 constexpr int kFwdSmallWaves = 4;
-constexpr int kFwdSmallMaxT = 1024;
+constexpr int kFwdSmallMaxT = 4096;
 // (at the end the area also takes the wave's partial O^T, 4 KiB per 32 columns of the head dim)
 constexpr int fwd_small_wave_bytes(int D, int dtype) {
     const int blocks = 2 * 32 * D * elem_bytes(dtype), partial = ((D + 31) / 32) * 16 * 64 * 4;
@@ -130,7 +138,8 @@ constexpr int fwd_small_wave_bytes(int D, int dtype) {
 }
 constexpr int fwd_small_lds_bytes(int D, int dtype) { return kFwdSmallWaves * fwd_small_wave_bytes(D, dtype); }
 constexpr bool fwd_takes_small(long long batch_heads, int T, int D, int dtype) {
-    return D * elem_bytes(dtype) <= 512 && T <= kFwdSmallMaxT && batch_heads * ((T + 127) / 128) <= kComputeUnits / 4;
+    return CHILL_TUNE_FWD_SMALL && D * elem_bytes(dtype) <= 512 && T <= kFwdSmallMaxT &&
+           batch_heads * ((T + 31) / 32) <= ((dtype == CHILL_F32 || D >= 128) ? 2 : 1) * kComputeUnits;
 }
 
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {

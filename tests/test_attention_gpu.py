@@ -79,11 +79,11 @@ def make_qkv(shape, dtype, noncontiguous):
 
 
 # (noncontiguous, head_dim, B, (H, H_kv)) combinations covering every value of the reference matrix
-# Launches of at most 64 workgroups' worth of rows at T <= 1024 take the forward that splits the keys of
-# a q-tile over its waves; (11, (6, 3)) keeps the ordinary forward covered at the short lengths, the
-# shapes with B = 1 cover the other one at the longer ones.
+# Launches of up to 256 or 512 q-tiles of 32 rows take the forward that splits the keys of a q-tile over
+# its waves; (87, (6, 3)) keeps the ordinary forward covered at the shortest lengths (it is left out at
+# the others), the shapes with B = 1 cover the other one at the longer ones.
 FWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (6, 3)), (False, 128, 1, (6, 1)), (True, 16, 7, (8, 8)),
-              (False, 64, 11, (6, 3))]
+              (False, 64, 87, (6, 3))]
 BWD_SHAPES = [(False, 16, 1, (1, 1)), (True, 128, 7, (8, 2)), (False, 128, 16, (6, 1)), (True, 16, 7, (8, 8)),
               (False, 128, 1, (8, 1))]
 
@@ -96,6 +96,8 @@ def test_forward_matrix(m, dtype, lens_kind, T):
     mask = make_mask(m)
     rng = np.random.default_rng(stable_seed(m, str(dtype), lens_kind, T))
     for noncontig, D, B, (H, Hkv) in FWD_SHAPES:
+        if B == 87 and T > 16:
+            continue
         print(f"fwd {mask} {dtype} lens={lens_kind} T={T} noncontig={noncontig} D={D} B={B} H={H}/{Hkv}", flush=True)
         q = make_qkv((B, H, T, D), dtype, noncontig)
         k = make_qkv((B, Hkv, T, D), dtype, noncontig)
@@ -153,8 +155,8 @@ def test_small_launch_forward(m, dtype):
         ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), lens)
         out, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens, return_lse=True)
         check_close(out * res_mask, ref, dtype, OUT_TOL[dtype], D, f"O small launch T={T} D={D}")
-        # the ordinary forward on the same rows: 40 copies of the batch make the launch large
-        rep = 40
+        # the ordinary forward on the same rows: copies of the batch make the launch large
+        rep = 40 if T > 100 else 200
         big, big_lse = ca.chill_attention(q.repeat(rep, 1, 1, 1), k.repeat(rep, 1, 1, 1), v.repeat(rep, 1, 1, 1),
                                           mask=mask, lens=lens.repeat(rep), return_lse=True)
         torch.testing.assert_close(out.float(), big[:B].float(), atol=OUT_TOL[dtype][0], rtol=OUT_TOL[dtype][1])
