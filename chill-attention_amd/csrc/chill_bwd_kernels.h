@@ -102,6 +102,10 @@ __device__ __forceinline__ void softmax_grad_block(f32x16& s, f32x16& dp, float 
     }
 }
 
+}  // namespace chill
+#include "chill_bwd_small.h"
+namespace chill {
+
 // ------------------------------------------------------------------------------------------ dQ
 // Same skeleton as the forward kernel: asynchronous K/V ring, 32-key steps, the two score GEMMs of
 // step t+1 (S^T and dP^T) issued before the vector work of step t.
@@ -379,6 +383,28 @@ int launch_dq_shape(const BwdParams& p, hipStream_t stream) {
     return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
 }
 
+// A launch far too small for the chip: 32 rows per workgroup, the streamed axis split over its waves.
+// PASS 1: dQ (workgroups over query blocks), 2: dK/dV (over key blocks).
+template <typename E, int D, int MASK_ID, int PASS>
+int launch_bwd_small(const BwdParams& p, hipStream_t stream) {
+    constexpr int kLdsBytes = bwd_small_lds_bytes(D, Elem<E>::kDType, PASS);
+    const int n_tiles = cdiv(p.T, 32);
+    const int total = p.B * (PASS == 1 ? p.H : p.H_kv) * n_tiles;  // (small by bwd_takes_small)
+    void (*kern)(BwdParams, int, int, int);
+    if constexpr (PASS == 1)
+        kern = dq_small_kernel<E, D, MASK_ID>;
+    else
+        kern = dkdv_small_kernel<E, D, MASK_ID>;
+    const bool hfb = Mask<MASK_ID>::has_full_blocks(32, 32, p.T, p.margs);
+    if (kLdsBytes > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsBytes) != hipSuccess)
+            return CHILL_ERR_HIP;
+    }
+    hipLaunchKernelGGL(kern, dim3(total), dim3(kFwdSmallWaves * 64), kLdsBytes, stream, p, n_tiles, total, hfb ? 1 : 0);
+    return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+}
+
 template <typename E, int D>
 int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
     const int64_t max_stride = p.sk.t > p.sv.t ? p.sk.t : p.sv.t;
@@ -388,7 +414,12 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
         // the table has a row of its own for short sequences and small grids where that row differs
         constexpr bool has_short_row = dq_tile_config(MASK_ID, D, Elem<E>::kDType, 1).waves !=
                                        dq_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
-        if constexpr (has_short_row) {
+        bool small = false;
+        constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DQ);
+        if constexpr (served) small = bwd_takes_small((long long)p.B * p.H, p.T, D, Elem<E>::kDType, CHILL_PASS_DQ);
+        if (small) {
+            if constexpr (served) status = launch_bwd_small<E, D, MASK_ID, 1>(p, stream);
+        } else if constexpr (has_short_row) {
             status = dq_takes_short_row((long long)p.B * p.H, p.T) ? launch_dq_shape<E, D, MASK_ID, true>(p, stream)
                                                                    : launch_dq_shape<E, D, MASK_ID, false>(p, stream);
         } else {
@@ -1120,7 +1151,12 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
         // the table has a row of its own for small grids where that row differs
         constexpr bool has_small_row = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, true).waves !=
                                        dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, false).waves;
-        if constexpr (has_small_row) {
+        bool small = false;
+        constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DKDV);
+        if constexpr (served) small = bwd_takes_small((long long)p.B * p.H_kv, p.T, D, Elem<E>::kDType, CHILL_PASS_DKDV);
+        if (small) {
+            if constexpr (served) status = launch_bwd_small<E, D, MASK_ID, 2>(p, stream);
+        } else if constexpr (has_small_row) {
             status = dkdv_takes_small_row((long long)p.B * p.H_kv, p.T) ? launch_dkdv_shape<E, D, MASK_ID, true>(p, stream)
                                                                         : launch_dkdv_shape<E, D, MASK_ID, false>(p, stream);
         } else {

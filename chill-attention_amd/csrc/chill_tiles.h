@@ -142,6 +142,34 @@ constexpr bool fwd_takes_small(long long batch_heads, int T, int D, int dtype) {
            batch_heads * ((T + 31) / 32) <= ((dtype == CHILL_F32 || D >= 128) ? 2 : 1) * kComputeUnits;
 }
 
+// The backward of such launches (dq_small_kernel, dkdv_small_kernel): the same split of the streamed
+// axis over four waves; a wave's area holds two 32-row blocks (K and V, or Q and dO), later its partial
+// accumulators (`outputs` x 4 KiB per 32 columns of the head dim), and LSE2 / delta of a query block.
+#ifndef CHILL_TUNE_BWD_SMALL
+#define CHILL_TUNE_BWD_SMALL 1
+#endif
+constexpr int bwd_small_wave_bytes(int D, int dtype, int outputs) {
+    const int blocks = 2 * 32 * D * elem_bytes(dtype), partial = outputs * ((D + 31) / 32) * 16 * 64 * 4;
+    return (blocks > partial ? blocks : partial) + 2 * 32 * 4;
+}
+constexpr int bwd_small_lds_bytes(int D, int dtype, int outputs) { return kFwdSmallWaves * bwd_small_wave_bytes(D, dtype, outputs); }
+#ifndef CHILL_TUNE_BWD_SMALL_SCALE
+#define CHILL_TUNE_BWD_SMALL_SCALE 1
+#endif
+// Where they win (measured against dq_kernel / dkdv_kernel on causal masks, 1 .. 128 heads, T = 128 .. 4096):
+// dQ while its grid of B * H * T / 32 workgroups is at most 512 (256 for 16-bit inputs at head dim 128):
+// 1.1x .. 1.9x for 16-bit inputs, 1.5x .. 3.8x for fp32; dK/dV at head dims up to 64 with at most 256 workgroups
+// (512 for fp32): 1.1x .. 1.4x and 1.2x .. 3.4x.  At head dim 128 dK/dV does not win (a wave then holds K, V and
+// two accumulators of 64 registers each), and fp32 rows of 512 bytes do not fit a wave's registers at all.
+constexpr bool bwd_small_serves(int D, int dtype, int pass) {
+    return CHILL_TUNE_BWD_SMALL && (pass == CHILL_PASS_DKDV ? D <= 64 : (D <= 128 && D * elem_bytes(dtype) <= 512));
+}
+constexpr bool bwd_takes_small(long long batch_heads, int T, int D, int dtype, int pass) {
+    const int chips = pass == CHILL_PASS_DKDV ? (dtype == CHILL_F32 ? 2 : 1) : ((dtype == CHILL_F32 || D <= 64) ? 2 : 1);
+    return bwd_small_serves(D, dtype, pass) && T <= kFwdSmallMaxT * CHILL_TUNE_BWD_SMALL_SCALE &&
+           batch_heads * ((T + 31) / 32) <= (long long)chips * kComputeUnits * CHILL_TUNE_BWD_SMALL_SCALE;
+}
+
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {
     const int waves = fwd_waves(mask_id, D, dtype, T);
     const int streamed = fwd_streamed(mask_id, D, dtype, T);
@@ -260,10 +288,18 @@ inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_
             *out = fwd_tile_config(mask_id, D, dtype, (T != kLongSequence && fwd_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
             return CHILL_OK;
         case CHILL_PASS_DQ:
+            if (T != kLongSequence && bwd_takes_small(batch_heads, T, D, dtype, CHILL_PASS_DQ)) {
+                *out = TileConfig{32, 32, kFwdSmallWaves, bwd_small_lds_bytes(D, dtype, 1)};
+                return CHILL_OK;
+            }
             *out = dq_tile_config(mask_id, D, dtype, (T != kLongSequence && dq_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
             return CHILL_OK;
         case CHILL_PASS_DKDV:
             // (for this pass batch_heads counts the key / value heads)
+            if (T != kLongSequence && bwd_takes_small(batch_heads, T, D, dtype, CHILL_PASS_DKDV)) {
+                *out = TileConfig{32, 32, kFwdSmallWaves, bwd_small_lds_bytes(D, dtype, 2)};
+                return CHILL_OK;
+            }
             *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T));
             return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
