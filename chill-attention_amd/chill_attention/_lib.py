@@ -128,8 +128,15 @@ def torch_operator():
         if os.environ.get("CHILL_ATTENTION_EAGER_OP", "1") != "0" and os.path.exists(TORCH_LIB_PATH):
             import torch
 
-            torch.ops.load_library(TORCH_LIB_PATH)
-            _torch_operator = torch.ops.chill_attention_amd.attention
+            try:
+                torch.ops.load_library(TORCH_LIB_PATH)
+                _torch_operator = torch.ops.chill_attention_amd.attention
+            except (OSError, RuntimeError) as e:
+                # built against another PyTorch: the torch.library operators do the same work
+                import warnings
+
+                warnings.warn(f"chill_attention: {TORCH_LIB_PATH} does not load ({e}); eager calls take the "
+                              "torch.library operators (rebuild with `make -C chill-attention_amd/csrc`)")
     return _torch_operator
 
 

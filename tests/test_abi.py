@@ -241,3 +241,18 @@ def test_hand_managed_accumulation_registers(elem):
             if kernel in name:
                 assert compiler_max < hand_min, (name, compiler_max, hand_min)
                 assert hand_min == lowest and spilled == 0, (name, hand_min, spilled)
+
+
+def test_eager_operator_library_loads():
+    """The operator registered from C++ (csrc/chill_torch.cpp) is built next to the kernel library, loads
+    into this PyTorch and has the schema the Python side calls it with."""
+    import torch
+
+    assert os.path.exists(_lib.TORCH_LIB_PATH), "libchill_attention_torch.so has not been built"
+    op = _lib.torch_operator()
+    assert op is not None
+    schema = str(torch.ops.chill_attention_amd.attention.default._schema)
+    assert schema == ("chill_attention_amd::attention(Tensor q, Tensor k, Tensor v, Tensor? lens, int entry_points, "
+                      "int mask_id, int[] mask_args, float sm_scale, bool return_lse) -> (Tensor, Tensor)")
+    table = _lib.entry_points(_lib.lib)
+    assert all(getattr(table, n) for n, _ in _lib.EntryPoints._fields_)
