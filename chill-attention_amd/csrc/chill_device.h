@@ -725,29 +725,50 @@ __device__ __forceinline__ void load_resident(Resident<E, D>& regs,
 
 // Store one output row from transposed accumulators: lane (n, h) holds, for every 32-wide block
 // db of the head dim, the 16 values of columns d = 32*db + 8*(r/4) + 4*h + r%4 of ITS row.
-// Each group of four consecutive r is four consecutive d, written as one 8- or 16-byte store.
-// Rows that are not `valid` are written as zeros.
+// Each group of four consecutive r is four consecutive d.  fp32: one 16-byte store per group.  16-bit
+// types: the two lanes of a row trade one 8-byte group of every pair (v_permlane32_swap), so that each
+// writes 16 contiguous bytes and a store instruction covers 32 contiguous bytes of every row (8-byte
+// stores scattered over 32 rows reach HBM as partial sectors: the forward wrote 1.33x its output).
+// Both lanes of a row must be active or inactive together.  Rows that are not `valid` are written as zeros.
 template <typename E, int D>
 __device__ __forceinline__ void store_row_transposed(typename Elem<E>::type* row_ptr,
                                                      const f32x16 (&acc)[(D + 31) / 32], float mult,
                                                      bool valid, int h) {
     constexpr int DB = (D + 31) / 32;
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+    for (int db = 0; db < DB; db++) {
+        if constexpr (Elem<E>::k16) {
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            int d0 = 32 * db + 8 * g + 4 * h;
-            if (D >= 32 || d0 < D) {
-                f32x4 vals;
+            for (int gp = 0; gp < 2; gp++) {
+                if (D >= 32 || 16 * gp < D) {
+                    f32x4 va, vb;
 #pragma unroll
-                for (int e = 0; e < 4; e++) vals[e] = valid ? acc[db][4 * g + e] * mult : 0.f;
-                if constexpr (Elem<E>::k16) {
-                    *reinterpret_cast<i32x2*>(row_ptr + d0) = Elem<E>::pack4(vals);
-                } else {
+                    for (int e = 0; e < 4; e++) {
+                        va[e] = valid ? acc[db][8 * gp + e] * mult : 0.f;
+                        vb[e] = valid ? acc[db][8 * gp + 4 + e] * mult : 0.f;
+                    }
+                    const i32x2 a = Elem<E>::pack4(va), b = Elem<E>::pack4(vb);
+                    // first: lanes h = 0 keep their group 2 gp, lanes h = 1 receive the partner's group 2 gp + 1;
+                    // second: lanes h = 0 receive the partner's group 2 gp, lanes h = 1 keep their group 2 gp + 1
+                    const auto w0 = __builtin_amdgcn_permlane32_swap(a[0], b[0], false, false);
+                    const auto w1 = __builtin_amdgcn_permlane32_swap(a[1], b[1], false, false);
+                    *reinterpret_cast<i32x4*>(row_ptr + 32 * db + 16 * gp + 8 * h) =
+                        i32x4{(int)w0[0], (int)w1[0], (int)w0[1], (int)w1[1]};
+                }
+            }
+        } else {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                int d0 = 32 * db + 8 * g + 4 * h;
+                if (D >= 32 || d0 < D) {
+                    f32x4 vals;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) vals[e] = valid ? acc[db][4 * g + e] * mult : 0.f;
                     *reinterpret_cast<f32x4*>(row_ptr + d0) = vals;
                 }
             }
         }
+    }
 }
 
 // Zero rows [row0, row0 + nrows) of a [T, D] slab (inner stride 1) cooperatively.
