@@ -357,11 +357,15 @@ void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
 }
 
 // One (mask, tile shape): SHORT selects the table row for short sequences.
+// (defined below, next to the kernel it is modelled on)
+template <typename E, int D, int MASK, int NW, int NS>
+__global__ void dq_split_kernel(BwdParams p, int n_q_tiles, int total_items, int wave_has_full_blocks);
+
 template <typename E, int D, int MASK_ID, bool SHORT>
 int launch_dq_shape(const BwdParams& p, hipStream_t stream) {
     constexpr int kRowFor = SHORT ? 1 : kLongSequence;
     constexpr TileConfig cfg = dq_tile_config(MASK_ID, D, Elem<E>::kDType, kRowFor);
-    static_assert(cfg.rows == cfg.waves * 32, "one wave owns 32 rows");
+    static_assert(cfg.rows == cfg.waves * (dq_is_split(D, Elem<E>::kDType) ? 16 : 32), "one wave (or a pair) owns 32 rows");
     constexpr int NS = dq_stages(MASK_ID, D, Elem<E>::kDType, kRowFor);
     const int n_q_tiles = cdiv(p.T, cfg.rows);
     const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
@@ -371,6 +375,8 @@ int launch_dq_shape(const BwdParams& p, hipStream_t stream) {
     void (*kern)(BwdParams, int, int, int);
     if constexpr (dq_regs_keys(D, Elem<E>::kDType) > 0)
         kern = dq_regs_kernel<E, D, MASK_ID, cfg.streamed, NS>;
+    else if constexpr (dq_is_split(D, Elem<E>::kDType))
+        kern = dq_split_kernel<E, D, MASK_ID, cfg.waves, NS>;
     else
         kern = dq_kernel<E, D, MASK_ID, cfg.waves, cfg.streamed, NS>;
     const bool hfb = Mask<MASK_ID>::has_full_blocks(32, cfg.streamed, p.T, p.margs);
@@ -427,6 +433,199 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
         }
     });
     return status;
+}
+
+// ------------------------------------------------------------------------------------------ dQ (wide rows)
+// fp32 rows of 1 KiB (head dim 256): a wave that owns 32 query rows would hold Q and dO as resident
+// operands (256 registers) and dQ^T (128): dq_kernel spilled 245 registers there.  Two waves share a
+// 32-query block instead, the way dkdv_split_kernel's waves share a key block: the even one holds Q and
+// computes S^T = K Q^T (scale and LSE2 applied), the odd one holds dO and computes dP^T = V dO^T - delta;
+// the two products meet in LDS, both waves compute P and dS, and each accumulates half of the head-dim
+// blocks of dQ^T += K^T dS^T.  No MFMA is issued twice and both waves issue the same number.
+template <typename E, int D, int MASK, int NW, int NS>
+__global__ __launch_bounds__(NW * 64) void dq_split_kernel(BwdParams p, int n_q_tiles, int total_items,
+                                                      int wave_has_full_blocks) {
+    using ET = typename Elem<E>::type;
+    typedef LdsTile<E, D> L;
+    static_assert(!Elem<E>::k16, "fp32 rows");
+    constexpr int TK = 32;
+    constexpr int NQB = NW / 2;       // 32-query blocks per workgroup
+    constexpr int TQ = NQB * 32;
+    constexpr int NT = NW * 64;
+    constexpr int DB = D / 32;
+    constexpr int DBW = DB / 2;       // head-dim blocks a wave accumulates
+    constexpr int NJ = L::CH / 2;
+    constexpr int TILE_BYTES = L::bytes(TK);
+    constexpr int STAGE_BYTES = 2 * TILE_BYTES;  // K tile, then V tile
+    constexpr int X_BYTES = 16 * 64 * 4;         // one product
+    static_assert(NS == 2, "two ring stages");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    if (item < 0) return;
+    const int bh = item / n_q_tiles;
+    const int qt = n_q_tiles - 1 - item % n_q_tiles;
+    const int b = bh / p.H;
+    const int hd = bh % p.H;
+    const int hkv = hd / p.group;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int qblk = wave % NQB;
+    const int role = wave / NQB;  // 0: S from Q, 1: dP from dO; also the half of the head dim it accumulates
+    const int n = lane & 31;
+    const int h = lane >> 5;
+
+    int seq_len = p.T;
+    if (p.lens != nullptr) seq_len = imin(p.lens[(int64_t)b * p.lens_stride], p.T);
+
+    const int qb = qt * TQ;
+    ET* dqbase = reinterpret_cast<ET*>(p.dq) + b * p.sdq.b + hd * p.sdq.h;
+    if (qb >= seq_len) {
+        zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(TQ, p.T - qb), tid);
+        return;
+    }
+
+    const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
+    const ET* vptr = reinterpret_cast<const ET*>(p.v) + b * p.sv.b + hkv * p.sv.h;
+    const TileRange wg = tile_range<MASK, true>(qb, TQ, TK, seq_len, false, p.margs);
+    const int n_tiles = wg.end - wg.start;
+    AsyncSwizzledLoader<E, D, TK, NT> load_k, load_v;
+    load_k.init(p.sk.t, wave, lane);
+    load_v.init(p.sv.t, wave, lane);
+    auto issue_tile = [&](int i, int st_index) {
+        int k0 = (wg.start + i) * TK;
+        char* st = smem + st_index * STAGE_BYTES;
+        load_k.issue(kptr + (int64_t)k0 * p.sk.t, p.T - k0, st, wave, lane);
+        load_v.issue(vptr + (int64_t)k0 * p.sv.t, p.T - k0, st + TILE_BYTES, wave, lane);
+    };
+    if (n_tiles > 0) issue_tile(0, 0);
+
+    // this wave's resident operand: the block's Q rows (role 0) or dO rows (role 1); LSE2 or delta of
+    // the lane's row
+    const int qw = qb + 32 * qblk;
+    const int q_pos = qw + n;
+    Resident<E, D> res;
+    float sub = 0.f;
+    {
+        const int64_t stride = role == 0 ? p.sq.t : p.sdo.t;
+        const ET* src = role == 0 ? reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hd * p.sq.h
+                                  : reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hd * p.sdo.h;
+        load_resident<E, D>(res, src + (int64_t)qw * stride, stride, p.T - qw, lane);
+        if (q_pos < p.T)
+            sub = role == 0 ? p.lse[b * p.lse_b + hd * p.lse_h + q_pos] : p.delta[b * p.delta_b + hd * p.delta_h + q_pos];
+        // a row that attends to nothing has LSE2 = -inf and only masked entries, which a select zeroes
+        if (role == 0 && sub == -INFINITY) sub = 0.f;
+    }
+
+    TileRange wr = {wg.start, wg.start, wg.start, wg.start};
+    if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32, TK, seq_len, wave_has_full_blocks != 0, p.margs);
+    const int ta = wr.start - wg.start, tb = wr.end - wg.start;
+    const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
+
+    f32x16 dq[DBW];
+#pragma unroll
+    for (int i = 0; i < DBW; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dq[i][r] = 0.f;
+    const float mult = role == 0 ? p.scale_log2 : 1.f;
+    const lds_char* lds0 = (const lds_char*)smem;
+    // the two products of block qblk: register r of lane l at ((r / 4) * 64 + l) * 16 + (r % 4) * 4
+    char* xblock = smem + 2 * STAGE_BYTES + qblk * 2 * X_BYTES;
+    const int db0 = role * DBW;
+
+    for (int it = 0; it < n_tiles; it++) {
+        wait_async_tiles();
+        __syncthreads();  // tile `it` is in LDS; every wave is done with the iteration before
+        if (it + 1 < n_tiles) issue_tile(it + 1, (it + 1) & 1);
+        const bool mine = it >= ta && it < tb;  // (the same for both waves of a block)
+        const lds_char* stage = lds0 + (it & 1) * STAGE_BYTES;
+        // LDS offsets are derived from these inside the iteration: kept across iterations they would
+        // take more registers than the few vector instructions that compute them save
+        int n_it = n, h_it = h;
+        asm volatile("" : "+v"(n_it), "+v"(h_it));
+        if (mine) {
+            // rows = keys 8 * (r / 4) + 4 * h + r % 4 of the tile, column n = query row
+            const lds_char* src = stage + role * TILE_BYTES;
+            f32x16 acc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const i32x4 a = *reinterpret_cast<const lds_i32x4*>(src + L::chunk_off(n_it, 2 * j + h_it));
+                acc = Elem<E>::mma(a, res.c[j], acc);
+            }
+            // s * scale - LSE2 (what the exponential takes, chill_bwd_dq.py:314) or dP - delta
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = acc[r] * mult - sub;
+            f32x4* out = reinterpret_cast<f32x4*>(xblock + role * X_BYTES);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++)
+                out[r4 * 64 + lane] = f32x4{acc[4 * r4], acc[4 * r4 + 1], acc[4 * r4 + 2], acc[4 * r4 + 3]};
+        }
+        // the first operands of the accumulation do not depend on the exchange
+        float a_k[2][DBW];
+        auto read_operands = [&](int r, int buf) {
+            const int rw = 8 * (r / 4) + 4 * h_it + (r % 4);
+#pragma unroll
+            for (int i = 0; i < DBW; i++)
+                a_k[buf][i] = *reinterpret_cast<const lds_float*>(stage + L::elem_off(rw, 32 * (db0 + i) + n_it));
+        };
+        if (mine) read_operands(0, 0);
+        __syncthreads();  // the products of this iteration are in LDS
+        if (!mine) continue;
+
+        f32x16 cs, cdp;
+        {
+            const f32x4* xs = reinterpret_cast<const f32x4*>(xblock);
+            const f32x4* xd = reinterpret_cast<const f32x4*>(xblock + X_BYTES);
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const f32x4 a = xs[r4 * 64 + lane], d = xd[r4 * 64 + lane];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    cs[4 * r4 + i] = a[i];
+                    cdp[4 * r4 + i] = d[i];
+                }
+            }
+        }
+        const bool full = (it >= fa) && (it < fb);
+        const int k0 = (wg.start + it) * TK;
+        // P = exp2(s * scale - LSE2), dS = P (dP - delta), dQ^T += K^T dS^T over this wave's head-dim
+        // blocks; register by register, so that the vector work and the LDS reads of one register run
+        // under the MFMAs of the one before
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float pv = fast_exp2(cs[r]);
+            if (!full) {
+                const int key = k0 + 8 * (r / 4) + 4 * h + (r % 4);
+                const bool ok = (q_pos < seq_len) && (key < seq_len) && Mask<MASK>::pred(q_pos, key, seq_len, p.margs);
+                pv = ok ? pv : 0.f;
+            }
+            const float ds = pv * cdp[r];
+            if (r + 1 < 16) read_operands(r + 1, (r + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < DBW; i++) dq[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_k[r & 1][i], ds, dq[i], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // lane (n, h) holds columns d = 32 * (db0 + i) + 8 * (r / 4) + 4 * h + r % 4 of ITS query row
+    if (q_pos < p.T) {
+        const bool valid = q_pos < seq_len;
+        float* row = reinterpret_cast<float*>(dqbase + (int64_t)q_pos * p.sdq.t);
+#pragma unroll
+        for (int i = 0; i < DBW; i++)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+                f32x4 a;
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[e] = valid ? dq[i][4 * g4 + e] * p.sm_scale : 0.f;
+                *reinterpret_cast<f32x4*>(row + 32 * (db0 + i) + 8 * g4 + 4 * h) = a;
+            }
+    }
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV

@@ -203,9 +203,13 @@ constexpr int dq_stages(int mask_id, int D, int dtype, int T) {
     return 3 * 2 * dq_streamed(D, dtype) * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
 }
 
+// fp32 at head dim 256 (dq_split_kernel): two waves share a 32-query block; two stages of 32-key K and V
+// tiles, then one 4 KiB slot per wave for the two products of a block.
+constexpr bool dq_is_split(int D, int dtype) { return dtype == CHILL_F32 && D == 256; }
 constexpr TileConfig dq_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {
     const int waves = dq_waves(mask_id, D, dtype, T);
     const int streamed = dq_streamed(D, dtype);
+    if (dq_is_split(D, dtype)) return TileConfig{waves * 16, 32, waves, 2 * 2 * 32 * D * 4 + waves * 16 * 64 * 4};
     return TileConfig{waves * 32, streamed, waves,
                       dq_stages(mask_id, D, dtype, T) * 2 * streamed * D * elem_bytes(dtype)};
 }
