@@ -1024,9 +1024,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
                 }
             }
         constexpr int ROWS_PER_STEP = 64 / CH;  // 4 (D = 128) .. 32 (D = 16)
+        // (what is derived from the lane index here is derived again, not kept from the prologue through
+        // the whole loop: at 256 registers that cost a slot in scratch memory)
+        int lane_e = threadIdx.x & 63;
+        asm volatile("" : "+v"(lane_e));
 #pragma unroll
         for (int row0 = 0; row0 < 32; row0 += ROWS_PER_STEP) {
-            const int row = row0 + lane / CH, c = lane % CH;
+            const int row = row0 + lane_e / CH, c = lane_e % CH;
             // PITCH is a multiple of 8 only: two 8-byte reads
             const i32x2 lo = *reinterpret_cast<const i32x2*>(stage + row * PITCH + c * 16);
             const i32x2 hi = *reinterpret_cast<const i32x2*>(stage + row * PITCH + c * 16 + 8);
