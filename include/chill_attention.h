@@ -203,8 +203,10 @@ int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, i
  * rows of 16-bit inputs use a smaller workgroup for short sequences and for grids that would not fill
  * the chip (the reference's tables, autotune.py:11-119, do not depend on the shape; its autotuner's key
  * does, autotune.py:129-240), and the dK/dV row one that covers half as many key rows for such grids
- * (batch_heads = B * H_kv for that pass).  chill_tile_config reports the row of long sequences on a
- * full chip. */
+ * (batch_heads = B * H_kv for that pass).  Launches far too small for the chip (a few hundred 32-row
+ * blocks in all) take kernels of their own, in which a workgroup owns 32 rows and its four waves split
+ * the streamed axis: reported as {32, 32, 4, lds_bytes}.  chill_tile_config reports the row of long
+ * sequences on a full chip. */
 int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
                                 int32_t T, int32_t out[4]);
 
