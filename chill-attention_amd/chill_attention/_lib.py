@@ -105,15 +105,35 @@ BWD_NOALLOC_MAX_ROWS = 4 * 1024 * 1024  # CHILL_BWD_NOALLOC_MAX_ROWS of the head
 TORCH_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libchill_attention_torch.so")
 
 
-class EntryPoints(ctypes.Structure):
-    """Addresses of one kernel library's entry points, in the order csrc/chill_torch.cpp declares."""
+ENTRY_POINTS_MAGIC = 0x4350454C4C494843  # "CHILLEPC", as csrc/chill_torch.cpp checks it
 
-    _fields_ = [(n, c_void_p) for n in ("fwd", "delta", "dkdv", "dq", "status_string")]
+
+class EntryPoints(ctypes.Structure):
+    """Addresses of one kernel library's entry points behind a magic word, the ABI version and the size
+    of the table, in the order csrc/chill_torch.cpp declares."""
+
+    _fields_ = [("magic", ctypes.c_uint64), ("abi_version", ctypes.c_uint32), ("bytes", ctypes.c_uint32)] + [
+        (n, c_void_p) for n in ("fwd", "delta", "dkdv", "dq", "status_string")]
 
 
 def entry_points(cdll: ctypes.CDLL) -> EntryPoints:
     names = ("chill_fwd", "chill_bwd_delta", "chill_bwd_dkdv", "chill_bwd_dq", "chill_status_string")
-    return EntryPoints(*(ctypes.cast(getattr(cdll, n), c_void_p).value for n in names))
+    return EntryPoints(ENTRY_POINTS_MAGIC, cdll.chill_abi_version(), ctypes.sizeof(EntryPoints),
+                       *(ctypes.cast(getattr(cdll, n), c_void_p).value for n in names))
+
+
+def register_entry_points(cdll: ctypes.CDLL) -> int:
+    """Hands the entry points of one kernel library to the C++ operator; returns the handle its calls name
+    the library by."""
+    assert torch_operator() is not None
+    reg = ctypes.CDLL(TORCH_LIB_PATH).chill_torch_register_entry_points
+    reg.argtypes, reg.restype = [c_void_p], ctypes.c_int64
+    table = entry_points(cdll)
+    handle = reg(ctypes.addressof(table))
+    if handle < 0:
+        raise RuntimeError(f"{TORCH_LIB_PATH} refuses the entry points of {cdll._name} "
+                           f"({'another ABI version' if handle == -2 else 'not a table'})")
+    return handle
 
 
 _torch_operator = False  # not looked for yet

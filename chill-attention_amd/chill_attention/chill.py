@@ -271,7 +271,7 @@ def _chill_reference_naive(
     return out * res_mask, res_mask
 
 
-# mask class -> (C++ operator or None, entry-point table of the class's kernel library, mask id)
+# mask class -> (C++ operator or None, the operator's handle of the class's kernel library, mask id)
 _eager = {}
 
 
@@ -282,7 +282,7 @@ def _eager_operator(mask: ChillMask):
         op = _lib.torch_operator()
         table = mask_id = None
         if op is not None:
-            table = _lib.entry_points(cls._library())
+            table = _lib.register_entry_points(cls._library())
             mask_id = _descriptor(cls, mask.constargs).id
         entry = _eager[cls] = (op, table, mask_id)
     return entry
@@ -338,7 +338,7 @@ def chill_attention(
             _check_inputs(q, k, v, lens, sm_scale)
             mask_args = [int(a) for a in mask.constargs]
             _require(all(a == b for a, b in zip(mask_args, mask.constargs)), "mask arguments must be integers")
-            O, LSE = op(q, k, v, lens, ctypes.addressof(table), mask_id, mask_args, float(sm_scale), bool(return_lse))
+            O, LSE = op(q, k, v, lens, table, mask_id, mask_args, float(sm_scale), bool(return_lse))
             return (O, LSE) if return_lse else O
     if not torch.compiler.is_compiling():
         for i in (q, k, v):

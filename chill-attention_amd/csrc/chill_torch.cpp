@@ -9,25 +9,47 @@
 // addresses of its entry points (the stock library's, or those of the library built around a
 // user-written mask), so one operator serves every mask class.
 //
-// Inputs are validated by the Python caller (chill.py, _check_inputs) before they get here.
+// The Python caller validates its inputs (chill.py, _check_inputs) with the reference's messages; the checks
+// that keep a direct call of the operator from crashing the process (devices, dtypes, shapes, the table of
+// entry points) are repeated here.
 #include <ATen/ATen.h>
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 #include <torch/csrc/autograd/custom_function.h>
 #include <torch/library.h>
 
+#include <cstring>
+#include <deque>
+#include <mutex>
+
 #include "../../include/chill_attention.h"
 
 namespace {
 
-// What `entry_points` points to: filled in by the Python side (ctypes) once per kernel library.
+// The entry points of one kernel library.  The Python side (ctypes) fills a table per library and registers
+// it once through chill_torch_register_entry_points; the operator takes the small handle that call returns,
+// never an address.
+constexpr uint64_t kEntryPointsMagic = 0x4350454c4c494843ull;  // "CHILLEPC"
 struct EntryPoints {
+    uint64_t magic;        // kEntryPointsMagic
+    uint32_t abi_version;  // CHILL_ABI_VERSION of the header the table was filled against
+    uint32_t bytes;        // sizeof(EntryPoints)
     decltype(&chill_fwd) fwd;
     decltype(&chill_bwd_delta) delta;
     decltype(&chill_bwd_dkdv) dkdv;
     decltype(&chill_bwd_dq) dq;
     decltype(&chill_status_string) status_string;
 };
+
+std::mutex g_tables_mutex;
+std::deque<EntryPoints> g_tables;  // (a deque: registered tables never move)
+
+const EntryPoints* table_of(int64_t handle) {
+    std::lock_guard<std::mutex> lock(g_tables_mutex);
+    TORCH_CHECK(handle >= 0 && handle < (int64_t)g_tables.size(), "chill_attention: ", handle,
+                " is not a handle of chill_torch_register_entry_points (", g_tables.size(), " registered)");
+    return &g_tables[(size_t)handle];
+}
 
 int32_t dtype_code(const at::Tensor& t) {
     switch (t.scalar_type()) {
@@ -67,11 +89,28 @@ void check(const EntryPoints* ep, const char* what, int status) {
     TORCH_CHECK(status >= 0, what, " failed with status ", status, ": ", ep->status_string(status));
 }
 
+// what the kernels assume of their operands and the C ABI cannot see from a raw pointer
+void check_operands(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const c10::optional<at::Tensor>& lens) {
+    TORCH_CHECK(q.is_cuda() && k.is_cuda() && v.is_cuda(), "chill_attention: q, k, v must be GPU tensors");
+    TORCH_CHECK(k.device() == q.device() && v.device() == q.device(), "chill_attention: q, k, v must be on one device");
+    TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4, "chill_attention: q, k, v must be [B, H, T, D]");
+    TORCH_CHECK(k.scalar_type() == q.scalar_type() && v.scalar_type() == q.scalar_type(),
+                "chill_attention: q, k, v must have one dtype");
+    TORCH_CHECK(k.sizes() == v.sizes() && k.size(0) == q.size(0) && k.size(2) == q.size(2) && k.size(3) == q.size(3),
+                "chill_attention: k, v must be [B, H_kv, T, D] for q of [B, H, T, D]");
+    TORCH_CHECK(k.size(1) > 0 && q.size(1) % k.size(1) == 0, "chill_attention: H must be a multiple of H_kv");
+    if (lens.has_value() && lens->defined())
+        TORCH_CHECK(lens->device() == q.device() && lens->scalar_type() == at::kInt && lens->dim() == 1 &&
+                        lens->size(0) == q.size(0),
+                    "chill_attention: lens must be an int32 tensor of [B] on the device of q");
+}
+
 std::tuple<at::Tensor, at::Tensor> forward_impl(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v,
                                                 const c10::optional<at::Tensor>& lens, int64_t entry_points,
                                                 int64_t mask_id, at::IntArrayRef mask_args, double sm_scale,
                                                 bool return_lse) {
-    const auto* ep = reinterpret_cast<const EntryPoints*>(entry_points);
+    const EntryPoints* ep = table_of(entry_points);
+    check_operands(q, k, v, lens);
     c10::DeviceGuard guard(q.device());
     const at::Tensor qv = kernel_view(q), kv = kernel_view(k), vv = kernel_view(v);
     // the kernel writes every row (zeros where nothing attends), so no zero fill is needed
@@ -95,7 +134,14 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> backward_impl(const at::Tensor& q
                                                              const at::Tensor& o, const at::Tensor& lse_in,
                                                              const at::Tensor& d_o, int64_t entry_points, int64_t mask_id,
                                                              at::IntArrayRef mask_args, double sm_scale) {
-    const auto* ep = reinterpret_cast<const EntryPoints*>(entry_points);
+    const EntryPoints* ep = table_of(entry_points);
+    check_operands(q, k, v, lens);
+    TORCH_CHECK(o.sizes() == q.sizes() && d_o.sizes() == q.sizes() && o.device() == q.device() && d_o.device() == q.device() &&
+                    o.scalar_type() == q.scalar_type(),
+                "chill_attention: o and its gradient must match q");
+    TORCH_CHECK(lse_in.device() == q.device() && lse_in.scalar_type() == at::kFloat && lse_in.dim() == 3 &&
+                    lse_in.size(0) == q.size(0) && lse_in.size(1) == q.size(1) && lse_in.size(2) == q.size(2),
+                "chill_attention: the saved LSE must be fp32 [B, H, T]");
     c10::DeviceGuard guard(q.device());
     const at::Tensor qv = kernel_view(q), kv = kernel_view(k), vv = kernel_view(v), ov = kernel_view(o);
     const at::Tensor dov = kernel_view(d_o.scalar_type() == q.scalar_type() ? d_o : d_o.to(q.scalar_type()));
@@ -134,7 +180,8 @@ class Attention : public torch::autograd::Function<Attention> {
                                                   int64_t mask_id, std::vector<int64_t> mask_args, double sm_scale,
                                                   bool return_lse) {
         at::AutoDispatchBelowADInplaceOrView below;
-        const bool needs_grad = q.requires_grad() || k.requires_grad() || v.requires_grad();
+        // (nothing is saved, and no LSE computed for it, where autograd is switched off)
+        const bool needs_grad = at::GradMode::is_enabled() && (q.requires_grad() || k.requires_grad() || v.requires_grad());
         auto [o, lse] = forward_impl(q, k, v, lens, entry_points, mask_id, mask_args, sm_scale, return_lse || needs_grad);
         if (needs_grad) {
             ctx->save_for_backward({q, k, v, o, lse, lens.has_value() && lens->defined() ? *lens : at::Tensor()});
@@ -167,6 +214,21 @@ std::tuple<at::Tensor, at::Tensor> attention_autograd(const at::Tensor& q, const
 }
 
 }  // namespace
+
+// Registers a table of entry points; returns its handle (>= 0), or -1 if the table is not one (wrong magic or
+// size) and -2 if it was filled against another version of the C ABI.
+extern "C" int64_t chill_torch_register_entry_points(const void* table) {
+    if (table == nullptr) return -1;
+    EntryPoints t;
+    std::memcpy(&t, table, sizeof(uint64_t) + 2 * sizeof(uint32_t));
+    if (t.magic != kEntryPointsMagic || t.bytes != sizeof(EntryPoints)) return -1;
+    if (t.abi_version != CHILL_ABI_VERSION) return -2;
+    std::memcpy(&t, table, sizeof(EntryPoints));
+    if (!t.fwd || !t.delta || !t.dkdv || !t.dq || !t.status_string) return -1;
+    std::lock_guard<std::mutex> lock(g_tables_mutex);
+    g_tables.push_back(t);
+    return (int64_t)g_tables.size() - 1;
+}
 
 TORCH_LIBRARY(chill_attention_amd, m) {
     m.def(

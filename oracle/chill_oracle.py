@@ -404,6 +404,22 @@ def lse2(name, args, q, k, lens=None, sm_scale=None):
     return attention_f64(name, args, q, k, k, lens=lens, sm_scale=sm_scale)["lse2"]
 
 
+def lse2_dense(name, args, q, k, lens=None, sm_scale=None):
+    """The same LSE2 as `lse2`, on torch tensors of any device, in float64 (for inputs too large for the
+    numpy textbook): [B, H, T]; -inf for rows without a visible key, rows >= lens included."""
+    import torch
+
+    if q.shape[1] != k.shape[1]:
+        k = k.repeat_interleave(q.shape[1] // k.shape[1], dim=1)
+    B, _, T, D = q.shape
+    scale = D ** -0.5 if sm_scale is None else sm_scale
+    lens_np = None if lens is None else lens.detach().cpu().numpy()
+    m = torch.from_numpy(np.array(_full_mask(name, args, B, T, lens_np))).to(q.device)
+    s = torch.einsum("bhqd,bhkd->bhqk", q.double(), k.double()) * scale
+    s = torch.where(m, s, torch.full_like(s, -math.inf))
+    return torch.logsumexp(s, dim=-1) * math.log2(math.e)
+
+
 def delta(o, do):
     """delta[b,h,t] = sum_d o*do in fp32-or-better (utils.py:190)."""
     return (np.asarray(o, dtype=np.float64) * np.asarray(do, dtype=np.float64)).sum(-1)

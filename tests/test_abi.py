@@ -255,4 +255,22 @@ def test_eager_operator_library_loads():
     assert schema == ("chill_attention_amd::attention(Tensor q, Tensor k, Tensor v, Tensor? lens, int entry_points, "
                       "int mask_id, int[] mask_args, float sm_scale, bool return_lse) -> (Tensor, Tensor)")
     table = _lib.entry_points(_lib.lib)
-    assert all(getattr(table, n) for n, _ in _lib.EntryPoints._fields_)
+    assert all(getattr(table, n) for n, *_ in _lib.EntryPoints._fields_)
+    # the operator takes a handle of a registered table, and tables that are not one are refused
+    import ctypes
+
+    reg = ctypes.CDLL(_lib.TORCH_LIB_PATH).chill_torch_register_entry_points
+    reg.argtypes, reg.restype = [ctypes.c_void_p], ctypes.c_int64
+    handle = _lib.register_entry_points(_lib.lib)
+    assert handle >= 0 and _lib.register_entry_points(_lib.lib) == handle + 1
+    bad = _lib.entry_points(_lib.lib)
+    bad.magic ^= 1
+    assert reg(ctypes.addressof(bad)) == -1 and reg(None) == -1
+    old = _lib.entry_points(_lib.lib)
+    old.abi_version += 1
+    assert reg(ctypes.addressof(old)) == -2
+    q = torch.zeros(1, 1, 8, 16)
+    with pytest.raises(RuntimeError, match="not a handle"):
+        op(q, q, q, None, handle + 1000, 1, [], 0.25, False)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        op(q, q, q, None, handle, 1, [], 0.25, False)  # CPU tensors: no kernel for them, no crash

@@ -16,6 +16,7 @@ import torch
 
 import chill_attention as ca
 from chill_attention import _lib
+from chill_attention.tiles import tile_config
 from conftest import MASK_INSTANCES, make_mask, mask_id
 from oracle import chill_oracle as orc
 
@@ -303,35 +304,122 @@ def test_lse_and_fully_masked_rows():
     assert torch.equal(o3, o4)
 
 
-@pytest.mark.gpu
-@pytest.mark.parametrize("D", [64, 128, 256])
-@pytest.mark.parametrize("dtype,growth", [(torch.float16, 60.0), (torch.bfloat16, 400.0), (torch.float32, 60.0)], ids=str)
-def test_reference_max_is_raised_along_the_keys(dtype, growth, D):
-    """Scores that grow by `growth` (log2 units) along the key axis: the forward's reference max has to be
-    raised many times per row (16-bit inputs: whenever a block's sum of P leaves the guarded range), in rows
-    whose two half-wave lanes see different sums.  Same bar as the other forward tests."""
+# Forward kernels by the route a launch takes: (rows, waves) that chill_tile_config_for_shape reports.
+#   (256, 8): the generated loop of 16-bit inputs at head dim 128 (fwd_fast_q_tiles; a q-tile whose sums leave the
+#             range of the reference-free softmax is voted on and computed again by fwd_q_tile on the same LDS ring)
+#   (128, 4): head dim 64, 16-bit: the generated loop of that shape, same vote; head dim 128 at T <= 1024, head dim 32,
+#             fp32: fwd_q_tile itself (16-bit: the guarded raise of the reference; fp32: the running max); head dim 256,
+#             16-bit: fwd_regs_kernel
+#   (32, 4):  fwd_small_kernel
+# drift: which query rows carry the direction the scores grow along ("all"; "low": the lower half of the sequence, which
+# in a paired launch is the SECOND q-tile of every pair; "high": the upper half, the first q-tile of every pair; "wave":
+# the 32 rows 160 .. 191 of every fourth block of 256 rows).
+RAMP_CASES = [
+    # id, dtype, D, B, H, H_kv, T, (rows, waves), masks, drift, lens
+    ("d128-loop-unpaired", torch.bfloat16, 128, 2, 8, 8, 2048, (256, 8), (0, 1), "all", None),
+    ("d128-loop-unpaired-f16", torch.float16, 128, 2, 8, 2, 2048, (256, 8), (0, 1), "all", None),
+    ("d128-loop-paired", torch.bfloat16, 128, 4, 16, 16, 2048, (256, 8), (1, 7), "all", None),
+    ("d128-loop-paired-f16", torch.float16, 128, 4, 16, 4, 2048, (256, 8), (0, 1), "all", None),
+    ("d128-loop-paired-second-only", torch.bfloat16, 128, 4, 16, 16, 2048, (256, 8), (0, 1, 7), "low", None),
+    ("d128-loop-paired-first-only", torch.float16, 128, 4, 16, 16, 2048, (256, 8), (0, 1), "high", None),
+    ("d128-loop-paired-one-wave", torch.bfloat16, 128, 4, 16, 16, 2048, (256, 8), (0, 1, 7), "wave", None),
+    ("d128-loop-paired-lens", torch.bfloat16, 128, 4, 16, 8, 2048, (256, 8), (0, 1, 7), "all", (2048, 1500, 300, 2047)),
+    ("d128-loop-paired-lens-f16", torch.float16, 128, 4, 16, 16, 2048, (256, 8), (1,), "low", (700, 2048, 1, 1025)),
+    ("d64-loop", torch.bfloat16, 64, 2, 8, 8, 1024, (128, 4), (0, 1, 4), "all", None),
+    ("d64-loop-f16", torch.float16, 64, 2, 8, 4, 1024, (128, 4), (0, 1, 4), "all", None),
+    ("d64-loop-paired-second-only", torch.float16, 64, 8, 16, 16, 2048, (128, 4), (0, 1, 7), "low", None),
+    ("d64-loop-paired-lens", torch.bfloat16, 64, 8, 16, 16, 2048, (128, 4), (1, 7), "wave", (2048, 3, 999, 1024, 2048, 1500, 64, 129)),
+    ("d128-short-row", torch.bfloat16, 128, 8, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("d128-short-row-f16", torch.float16, 128, 8, 8, 8, 1024, (128, 4), (0, 1, 4), "wave", None),
+    ("d32", torch.float16, 32, 2, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("d32-bf16", torch.bfloat16, 32, 2, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("d256-regs", torch.bfloat16, 256, 2, 8, 8, 2048, (128, 4), (0, 1), "all", None),
+    ("d256-regs-f16", torch.float16, 256, 2, 8, 8, 2048, (128, 4), (0, 1, 7), "wave", None),
+    ("f32-d64", torch.float32, 64, 4, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("f32-d128", torch.float32, 128, 4, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("small-d64", torch.bfloat16, 64, 1, 2, 2, 1024, (32, 4), (0, 1), "all", None),
+    ("small-d128-f16", torch.float16, 128, 1, 2, 2, 1024, (32, 4), (0, 1), "all", None),
+    ("small-d256", torch.bfloat16, 256, 1, 2, 2, 1024, (32, 4), (0, 1), "all", None),
+]
+# what a row's scores have to rise by over its first keys (log2 units) before the reference-free softmax of the
+# generated loops leaves its range (chill_fwd_fast.h: bf16 l > 2^60; fp16 one block sum > 2^15, which a row sum above
+# 2^21 implies for up to 64 blocks), and what the test feeds
+RAMP_TRIP = {torch.bfloat16: 60.0, torch.float16: 21.0, torch.float32: 0.0}
+RAMP_GROWTH = {torch.bfloat16: 400.0, torch.float16: 60.0, torch.float32: 60.0}
+
+
+@pytest.mark.parametrize("case", RAMP_CASES, ids=lambda c: c[0])
+def test_reference_max_is_raised_along_the_keys(case):
+    """Scores that grow by RAMP_GROWTH (log2 units) along the key axis, for the rows selected by `drift`: the
+    forward's reference max has to follow them.  Every forward kernel has its own way (running max; a guarded raise;
+    the reference-free softmax of the generated loops, whose q-tiles are then voted on and computed again by
+    fwd_q_tile): one case per kernel and way, with the route asserted from the tile table.  O and LSE2 against the
+    oracle (chill_fwd.py:188-286 is the running-max softmax all of them must equal)."""
+    _, dtype, D, B, H, Hkv, T, route, mask_ix, drift, lens = case
+    growth = RAMP_GROWTH[dtype]
     torch.manual_seed(7)
-    B, H, T = 1, 2, 1024
     q = torch.randn(B, H, T, D, device=DEV) * 0.5
-    k = torch.randn(B, H, T, D, device=DEV) * 0.5
-    v = torch.randn(B, H, T, D, device=DEV)
+    k = torch.randn(B, Hkv, T, D, device=DEV) * 0.5
+    v = torch.randn(B, Hkv, T, D, device=DEV)
     # a common direction whose weight in k grows with the key position: score(q, k_t) ~ t * growth / T (log2 units)
+    # for the rows that carry it; the other rows have no component along it at all
     u = torch.nn.functional.normalize(torch.randn(D, device=DEV), dim=0)
-    q = q + 4.0 * u
+    rows = torch.arange(T, device=DEV)
+    carries = {"all": rows >= 0, "low": rows < T // 2, "high": rows >= T // 2,
+               "wave": ((rows // 256) % 4 == 3) & ((rows % 256) // 32 == 5)}[drift]
+    q = q - (q @ u)[..., None] * u
+    q = q + 4.0 * carries[None, None, :, None] * u
     ramp = torch.arange(T, device=DEV, dtype=torch.float32) / T
     k = k + (growth * (D ** 0.5) / (4.0 * 1.4427)) * ramp[None, None, :, None] * u
     q, k, v = (x.to(dtype) for x in (q, k, v))
-    for m in (MASK_INSTANCES[0], MASK_INSTANCES[1]):
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    for m in (MASK_INSTANCES[i] for i in mask_ix):
         mask = make_mask(m)
-        ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), None)
-        out, lse = ca.chill_attention(q, k, v, mask=mask, return_lse=True)
+        cfg = tile_config(mask, D, dtype, _lib.PASS_FWD, seq_len=T, batch_heads=B * H)
+        assert (cfg["rows"], cfg["waves"]) == route, f"{m}: this shape is served by {cfg}, the case is meant for {route}"
+        print(f"ramp {case[0]} {mask}: {cfg}", flush=True)
+        ref, res_mask = orc.reference_naive(m[0], m[1], q.float(), k.float(), v.float(), lens_t)
+        want_lse = orc.lse2_dense(m[0], m[1], q, k, lens_t)
+        if RAMP_TRIP[dtype] > 0:
+            # the inputs do what the case is for: in rows that carry the direction the exponent rises by more than the
+            # reference-free softmax can hold above ANY reference taken from a row's first 64 keys (every mask here
+            # starts its rows at key 0; LSE2 >= the largest exponent; the exponent of the first keys is below
+            # growth * 64 / T plus the noise of the other directions, a fraction of a unit)
+            risen = want_lse - growth * 64.0 / T - 4.0 > RAMP_TRIP[dtype]
+            hit = risen & carries[None, None, :]
+            assert hit.any(), "no row leaves the range"
+            if drift != "all":
+                quiet = want_lse[:, :, ~carries]
+                quiet = quiet[torch.isfinite(quiet)]
+                assert quiet.max() < 14.0 and quiet.min() > -6.0, "rows without the direction must stay inside the range"
+        out, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens_t, return_lse=True)
         atol, rtol = OUT_TOL[dtype]
         if dtype == torch.float32:
             # raw scores reach several hundred here: their fp32 rounding alone moves P by ~3e-5 relative, whatever
             # the order of the sums, so the fp32 bar of the other tests (2e-6 / 1e-4) is out of reach for both sides
             atol, rtol = 1e-5, 1e-3
-        assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+        assert torch.isfinite(out).all()
         torch.testing.assert_close(out * res_mask, ref.to(dtype), atol=atol, rtol=rtol)
+        # LSE2 (up to `growth` in size): rows inside lens that see a key; the rest is 0 or -inf by definition
+        seen = torch.isfinite(want_lse)
+        assert torch.isfinite(lse[seen]).all()
+        tight = 1e-2 if dtype != torch.float32 else 1e-3
+        err = (lse.double() - want_lse).abs()
+        if dtype != torch.float32 and D in (64, 128) and route != (32, 4) and not (D == 128 and route == (128, 4)):
+            # The generated loops take Q already multiplied by scale * log2(e) and rounded to the input type (what the
+            # reference's PRESCALE_QK does, chill_fwd.py:120-127, chill_bwd_dkdv.py:118): the exponent of a (query, key)
+            # pair then carries the rounding errors of D products, each up to eps * |q_d * k_d| * scale * log2(e): four
+            # standard deviations of their sum for independent roundings are allowed here.  (The keys of this test
+            # reach a norm of several hundred.)  Rows that leave the range are computed again from the unrounded Q
+            # and meet the tight bar.
+            eps = {torch.bfloat16: 2.0 ** -9, torch.float16: 2.0 ** -12}[dtype]
+            k_norm = k.float().norm(dim=-1).amax(dim=-1)  # [B, H_kv]
+            k_norm = k_norm.repeat_interleave(H // Hkv, dim=1)[..., None]
+            loose = 4.0 * eps * (D ** -0.5 * 1.4427) * q.float().norm(dim=-1) * k_norm / D ** 0.5
+            assert (err[seen & risen] <= tight + 1e-4 * want_lse[seen & risen].abs()).all(), err[seen & risen].max()
+            assert (err[seen] <= (tight + loose)[seen]).all(), (err - loose)[seen].max()
+        else:
+            assert (err[seen] <= tight + 1e-4 * want_lse[seen].abs()).all(), err[seen].max()
 
 
 def test_rows_without_keys():

@@ -247,3 +247,24 @@ def test_attention_invariants():
     r2 = orc.attention_f64(name, args, q, k, v, do, lens=np.array([33, 5]))
     assert (r2["o"][1, :, 5:] == 0).all() and np.isneginf(r2["lse2"][1, :, 5:]).all()
     assert (r2["dq"][1, :, 5:] == 0).all() and (r2["dk"][1, :, 5:] == 0).all() and (r2["dv"][1, :, 5:] == 0).all()
+
+
+def test_lse2_dense_equals_the_direct_sum():
+    """lse2_dense (torch, any device) against log2 of the plain sum of 2^(scaled score) over the visible
+    keys, written without a max (small scores), with GQA and lens; and against the numpy textbook."""
+    name, args = "ChunkwiseChillMask", (5, 1)
+    q, k, _, _ = _rand(2, 4, 2, 21, 8, seed=11)
+    lens = torch.tensor([21, 9], dtype=torch.int32)
+    got = orc.lse2_dense(name, args, q, k, lens).numpy()
+    dense = orc.dense_mask(name, args, 21)
+    want = np.full((2, 4, 21), -np.inf)
+    for b in range(2):
+        for h in range(4):
+            for i in range(int(lens[b])):
+                tot = 0.0
+                for j in range(int(lens[b])):
+                    if dense[i, j]:
+                        tot += 2.0 ** (float(q[b, h, i].double() @ k[b, h // 2, j].double()) * 8 ** -0.5 * math.log2(math.e))
+                want[b, h, i] = math.log2(tot)
+    np.testing.assert_allclose(got, want, atol=1e-10)
+    np.testing.assert_allclose(got, orc.lse2(name, args, q.numpy(), k.numpy(), lens=lens.numpy()), atol=1e-10)
