@@ -120,6 +120,44 @@ def make_inputs(torch, B, H, T, D, dtype, seed, sigma, device):
     return [t.to(dtype).to(device) for t in ts]  # q, k, v, dO
 
 
+def recomputed_q_tiles(torch, ca, mask, q, k, T, D, dname, heads=4):
+    """Fraction of the forward's q-tiles that the kernel computes twice, from a host-side model of its
+    test on `heads` (batch, head) slices: a row takes the max of the first 32-key block its wave visits as
+    reference m0 and the q-tile is done again if a row's sum of 2^(s - m0) leaves [2^-60, 2^60] (fp16:
+    falls below 2^-6, or the sixteen entries a lane holds of one block sum to more than 2^15)."""
+    from chill_attention import _lib
+    from chill_attention.tiles import tile_config
+
+    dtype = q.dtype
+    B, H = q.shape[:2]
+    rows = tile_config(mask, D, dtype, _lib.PASS_FWD, seq_len=T, batch_heads=B * H)["rows"]
+    dense = mask.make_mask(T).to(q.device)  # [T, T] bool
+    c = D ** -0.5 * 1.4426950408889634
+    first_key = dense.float().argmax(dim=1)  # first visible key of a row
+    first_block = first_key.view(T // 32, 32).amin(dim=1) // 32  # first block of the wave that owns the row
+    first_block = first_block.repeat_interleave(32)
+    cols = torch.arange(T, device=q.device)
+    in_first = (cols[None, :] // 32) == first_block[:, None]
+    lo, hi = (2.0 ** -60, 2.0 ** 60) if dname == "bf16" else (2.0 ** -6, 2.0 ** 60)
+    bad_tiles = total = 0
+    for i in range(heads):
+        b, h = (i * 7) % B, (i * 5) % H
+        hk = h // (H // k.shape[1])
+        s2 = ((q[b, h].float() * c).to(dtype).float() @ k[b, hk].float().T).masked_fill(~dense, float("-inf"))
+        m0 = s2.masked_fill(~in_first, float("-inf")).amax(dim=1)
+        m0 = torch.where(torch.isfinite(m0), m0, torch.zeros_like(m0))
+        p = torch.exp2(s2 - m0[:, None])
+        l = p.sum(dim=1)
+        bad = ~((l >= lo) & (l <= hi))
+        if dname == "f16":
+            # a lane holds keys 8 * j + 4 * half + (0 .. 3), j = 0 .. 3, of a block
+            lane_sums = p.view(T, T // 32, 4, 2, 4).sum(dim=(2, 4))
+            bad |= (lane_sums > 32768.0).any(dim=2).any(dim=1)
+        bad_tiles += int(bad.view(T // rows, rows).any(dim=1).sum())
+        total += T // rows
+    return {"fraction": bad_tiles / total, "q_tiles_sampled": total, "rows_per_q_tile": rows}
+
+
 class Runner:
     """Pre-allocated buffers + raw C-ABI launches for one workload."""
 
@@ -233,6 +271,12 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sustained-seconds", type=float, default=3.0,
                     help="length of the continuous loop behind the `sustained` figure (0: leave it out)")
+    ap.add_argument("--sigma", type=float, default=None,
+                    help="standard deviation of q, k, v, dO instead of the workload's (inspection: the forward of "
+                         "16-bit inputs at head dims 64 and 128 computes a q-tile twice when a row's softmax sum "
+                         "leaves the range its reference-free loop is exact in; the line then carries "
+                         "`fwd_recomputed_q_tiles`)")
+    ap.add_argument("--dtype", default=None, choices=["f32", "f16", "bf16"], help="element type instead of the workload's")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch one plain 1 GiB device copy (1 GiB read + 1 GiB written) before the warm-up: "
                          "the known-size dispatch that scales the FETCH_SIZE / WRITE_SIZE counters of a "
@@ -250,6 +294,10 @@ def main():
         sys.exit("bench.py: no GPU visible")
     mask_name, margs, dname, B, H, T, D, seed, sigma = WORKLOADS[args.workload]
     mode = "fwd" if args.workload == "C1" else args.mode
+    if args.sigma is not None:
+        sigma = args.sigma
+    if args.dtype is not None:
+        dname = args.dtype
     dtype = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dname]
     mask = getattr(ca, mask_name)(*margs)
     dev = torch.device("cuda:0")
@@ -339,25 +387,29 @@ def main():
     es = 4 if dname == "f32" else 2
     dom = max(range(len(kernels)), key=lambda i: k_ms[i])
     dom_name = kernels[dom][0]
-    if dom_name == "chill_bwd_delta":
-        alg = 2.0 * B * H * T * D * es + 4.0 * B * H * T
-        roof = {"kernel": dom_name, "bound": "hbm", "achieved": alg / (k_ms[dom] * 1e-3) / 1e9, "peak": PEAK_HBM_GBS,
-                "unit": "GB/s"}
+    alg_bytes = {
+        "chill_fwd": 4.0 * B * H * T * D * es + 4.0 * B * H * T,
+        "chill_bwd_delta": 2.0 * B * H * T * D * es + 4.0 * B * H * T,
+        "chill_bwd_dkdv": 6.0 * B * H * T * D * es + 8.0 * B * H * T,
+        "chill_bwd_dq": 5.0 * B * H * T * D * es + 8.0 * B * H * T,
+    }
+    alg_flops = per_entry[dom_name] * B * H * D * nnz
+    # the roof that bounds the kernel: max(FLOPs / peak, algorithmic bytes / HBM bandwidth)
+    t_mfma = alg_flops / (peak * 1e12)
+    t_hbm = alg_bytes[dom_name] / (PEAK_HBM_GBS * 1e9)
+    if t_hbm >= t_mfma:
+        roof = {"kernel": dom_name, "bound": "hbm", "achieved": alg_bytes[dom_name] / (k_ms[dom] * 1e-3) / 1e9,
+                "peak": PEAK_HBM_GBS, "unit": "GB/s"}
     else:
-        alg = per_entry[dom_name] * B * H * D * nnz
-        roof = {"kernel": dom_name, "bound": "mfma", "achieved": alg / (k_ms[dom] * 1e-3) / 1e12, "peak": peak,
+        roof = {"kernel": dom_name, "bound": "mfma", "achieved": alg_flops / (k_ms[dom] * 1e-3) / 1e12, "peak": peak,
                 "unit": "TFLOP/s"}
+    roof["bound_ms"] = {"mfma": t_mfma * 1e3, "hbm": t_hbm * 1e3}
     roof["frac"] = roof["achieved"] / roof["peak"]
     current = traffic_is_current()
     roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, dom_name)) if current else None
     roof["traffic_unit"] = "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, copy-scaled)"
     roof["traffic_source"] = TRAFFIC_SOURCE if current else f"none: {TRAFFIC_SOURCE} was measured on other kernel sources"
-    roof["algorithmic_bytes"] = {
-        "chill_fwd": 4.0 * B * H * T * D * es + 4.0 * B * H * T,
-        "chill_bwd_delta": 2.0 * B * H * T * D * es + 4.0 * B * H * T,
-        "chill_bwd_dkdv": 6.0 * B * H * T * D * es + 8.0 * B * H * T,
-        "chill_bwd_dq": 5.0 * B * H * T * D * es + 8.0 * B * H * T,
-    }[dom_name]
+    roof["algorithmic_bytes"] = alg_bytes[dom_name]
     roof["avg_launch_ms"] = k_ms[dom]
 
     out = {
@@ -382,11 +434,17 @@ def main():
         "fwd_tflops": fwd_flops / (k_ms[0] * 1e-3) / 1e12,
         "fwd_frac_of_peak": fwd_flops / (k_ms[0] * 1e-3) / 1e12 / peak,
         "roofline": roof,
+        "kernel_frac_of_own_roof": {
+            kernels[i][0]: max(per_entry[kernels[i][0]] * B * H * D * nnz / (peak * 1e12),
+                               alg_bytes[kernels[i][0]] / (PEAK_HBM_GBS * 1e9)) / (k_ms[i] * 1e-3)
+            for i in range(len(kernels))},
         "sustained": sustained,
         "sm_clock_mhz": sustained["sm_clock_mhz"] if sustained else None,
         "operator_ms_per_step": op_ms,
         "kernel_sources_digest": kernel_sources_digest(),
     }
+    if args.sigma is not None and dname != "f32" and D in (64, 128):
+        out["fwd_recomputed_q_tiles"] = recomputed_q_tiles(torch, ca, mask, q, k, T, D, dname)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, mask_name, margs, dname, T, D, mode, seed, sigma)
     print(json.dumps(out))

@@ -176,13 +176,6 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
         load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
     };
     prefetch(qt_a);
-#ifdef CHILL_FWD_TIMING
-    // instrumented build: wave 0 leaves 100 MHz timestamps of its phases in the LSE rows of its q-tile
-    unsigned stamps[8];
-#define CHILL_STAMP(i) stamps[i] = (unsigned)__builtin_amdgcn_s_memrealtime()
-#else
-#define CHILL_STAMP(i)
-#endif
 
 #pragma nounroll
     for (int item = 0; item < 2; item++) {
@@ -196,15 +189,9 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
             zero_rows<E, D, NT>(obase, p.so.t, qb, nrows, tid);
             if (lse_base)
                 for (int i = tid; i < nrows; i += NT) lse_base[qb + i] = 0.f;
-#ifndef CHILL_FWD_NO_PREFETCH
             if (qt_next >= 0) prefetch(qt_next);
-#endif
             continue;
         }
-        CHILL_STAMP(0);
-#ifdef CHILL_FWD_NO_PREFETCH
-        if (item > 0) prefetch(qt);
-#endif
         const TileRange wg = {uniform(wg_pre.start), uniform(wg_pre.end), 0, 0};
         const int n_tiles = wg.end - wg.start;
         const int qw = qb + 32 * wave;
@@ -255,7 +242,6 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
         f32x16 mneg;  // the accumulator block the score chains start from: -m0 everywhere
 #pragma unroll
         for (int r = 0; r < 16; r++) mneg[r] = 0.f;
-        CHILL_STAMP(1);
 
         bool have_ref = false;  // wave-uniform: the rows have their reference
         // One step outside the generated loop, from the scores to O: block g of the wave (the first one
@@ -339,14 +325,9 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
         };
         int i = 0;
         for (; i < i_lo || (i_lo == i_hi && i < n_tiles); i++) plain_tile(i);
-        CHILL_STAMP(2);
         if constexpr (fwd_has_generated_loop<E, D, NW, NS>()) {
             if (i_hi > i_lo) {
                 ring_top(i_lo, false);  // the generated loop issues the tile that is due here
-                CHILL_STAMP(3);
-#ifdef CHILL_FWD_TIMING
-                const unsigned clk0 = (unsigned)__builtin_amdgcn_s_memtime();
-#endif
                 if (!have_ref) {
                     // the wave starts here: the reference comes from its first block, whose scores the
                     // loop computes again
@@ -405,25 +386,17 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
                                               load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
                 }
                 if (Lim::kBlockLimit) over |= ((over_mask >> lane) & 1) != 0;
-                CHILL_STAMP(4);
-#ifdef CHILL_FWD_TIMING
-                stamps[1] = (unsigned)__builtin_amdgcn_s_memtime() - clk0;  // shader clocks spent in the loop
-#endif
                 st_cur = (st_cur + (i_hi - i_lo - 1)) % NS;
                 i = i_hi;
             }
         }
         for (; i < n_tiles; i++) plain_tile(i);
-        CHILL_STAMP(5);
 
         // the ring is free once every wave is here: start on the next q-tile before this one is stored
-#ifndef CHILL_FWD_NO_PREFETCH
         if (qt_next >= 0) {
             __syncthreads();
             prefetch(qt_next);
         }
-#endif
-        CHILL_STAMP(6);
 
         // epilogue: O = acc / l, LSE2 = m0 + log2(l) (chill_fwd.py:288-289, 327-328)
         const float l_tot = sum_across_halves(l_run);
@@ -440,16 +413,6 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
         // a row that sees keys must end with a sum inside the range (a NaN fails the comparison too)
         const bool bad = (vis.lo <= vis.hi) && (over || !(l_tot >= Lim::kLo && l_tot <= Lim::kHi));
         const bool again = __builtin_amdgcn_ballot_w64(bad) != 0;
-#ifdef CHILL_FWD_TIMING
-        CHILL_STAMP(7);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (wave == 0 && lane == 0 && lse_base != nullptr && qb + 9 <= p.T) {
-            unsigned end = (unsigned)__builtin_amdgcn_s_memrealtime();
-#pragma unroll
-            for (int t = 0; t < 8; t++) lse_base[qb + t] = __builtin_bit_cast(float, stamps[t]);
-            lse_base[qb + 8] = __builtin_bit_cast(float, end);
-        }
-#endif
         if (workgroup_any<NW>(again, smem + NS * Lds::STAGE_BYTES)) {
             // rare: give the ring to the kernel whose softmax follows the running max, then start over on
             // the next q-tile
@@ -457,12 +420,9 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
             __syncthreads();
             fwd_q_tile<E, D, MASK, NW, TK, 3>(p, smem, b, hd, qt, wave_has_full_blocks);
             __syncthreads();
-#ifndef CHILL_FWD_NO_PREFETCH
             if (qt_next >= 0) prefetch(qt_next);
-#endif
         }
     }
-#undef CHILL_STAMP
 }
 
 }  // namespace chill

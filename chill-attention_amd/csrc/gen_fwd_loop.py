@@ -312,7 +312,7 @@ def issue_ops(c: Config, st: Stream):
                 A("s_nop 0", "nop")
                 A(f"global_load_lds_dwordx4 {vr(gbase + j)}, s[{PTR_SGPR[ptr]}:{PTR_SGPR[ptr] + 1}]", "vmem", [gbase + j])
                 if partial:
-                    A("s_mov_b64 exec, -1", "salu")
+                    A("s_mov_b64 exec, %[execsave]", "salu")
             ops.append(load)
         lo, hi = f"s{PTR_SGPR[ptr]}", f"s{PTR_SGPR[ptr] + 1}"
 
@@ -461,11 +461,13 @@ def gen_loop(c: Config):
     head.add(f"v_add_u32 {vr(c.KA)}, %[tnext], {vr(c.KLANE)}", "valu", [c.KLANE], [c.KA])
     head.add(f"v_add_u32 {vr(c.VA[0])}, %[cur], {vr(c.VLANE)}", "valu", [c.VLANE], [c.VA[0]])
     head.add(f"v_add_u32 {vr(c.VA[1])}, %[tnext], {vr(c.VLANE)}", "valu", [c.VLANE], [c.VA[1]])
-    # EXEC of the loads of the last round: all lanes for the waves that have a slab in it
+    # EXEC of the loads of the last round: the lanes of the caller for the waves that have a slab in it, none
+    # for the others; the statement leaves EXEC as it found it
+    head.add("s_mov_b64 %[execsave], exec", "salu")
     head.add(f"s_cmp_lt_u32 %[wave], {c.kslabs - (c.kper - 1) * c.NW}", "salu")
-    head.add("s_cselect_b64 %[klast], -1, 0", "salu")
+    head.add("s_cselect_b64 %[klast], %[execsave], 0", "salu")
     head.add(f"s_cmp_lt_u32 %[wave], {c.vslabs - (c.vper - 1) * c.NW}", "salu")
-    head.add("s_cselect_b64 %[vlast], -1, 0", "salu")
+    head.add("s_cselect_b64 %[vlast], %[execsave], 0", "salu")
     gen_fill(c, fill)
     # fast tile: the pending loads under step 0, the rotation under step 1 (the K address of the next
     # tile behind the last K read of step 1), then only the wait and the barrier between tiles
@@ -517,6 +519,62 @@ def gen_loop(c: Config):
     return out.ins
 
 
+# scalar temporaries of the statement, and the special registers it writes (EXEC is saved and restored)
+TEMP_SGPRS = ("tfill", "tnext", "tm0", "ringend", "klast", "vlast", "execsave")
+SPECIAL_CLOBBERS = ["vcc", "scc", "m0"]
+
+
+def check_clobbers(ins, outs, clobbers, what):
+    """Everything the statement writes is an output operand or a clobber: vector registers from the
+    bookkeeping of the stream, scalar destinations from the text (named operands %[x] must be outputs;
+    physical and special registers must be clobbers or tied output registers)."""
+    import re
+
+    out_names = {n for n, _ in outs}
+    out_regs = set()
+    for _, cs in outs:
+        m = re.search(r"\{v\[(\d+):(\d+)\]\}", cs)
+        if m:
+            out_regs |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+        m = re.search(r"\{v(\d+)\}", cs)
+        if m:
+            out_regs.add(int(m.group(1)))
+    out_sregs = set()
+    for _, cs in outs:
+        m = re.search(r"\{s\[(\d+):(\d+)\]\}", cs)
+        if m:
+            out_sregs |= {f"s{r}" for r in range(int(m.group(1)), int(m.group(2)) + 1)}
+    clob_v = {int(x[1:]) for x in clobbers if re.fullmatch(r"v\d+", x)}
+    for i in ins:
+        for reg in i["writes"]:
+            if reg not in out_regs and reg not in clob_v:
+                raise SystemExit(f"{what}: '{i['text']}' writes v{reg}, which is neither an output nor a clobber")
+        if i["kind"] != "salu" and not i["text"].startswith("v_cmp"):
+            continue
+        parts = i["text"].split(None, 1)
+        if len(parts) < 2 or parts[0] in ("s_barrier", "s_branch", "s_nop") or parts[0].startswith("s_cbranch"):
+            continue
+        dest = parts[1].split(",")[0].strip()
+        if parts[0].startswith("s_cmp"):
+            dest = "scc"
+        m = re.fullmatch(r"%\[(\w+)\]", dest)
+        if m:
+            if m.group(1) not in out_names:
+                raise SystemExit(f"{what}: '{i['text']}' writes the input operand {dest}")
+            continue
+        if dest == "exec":
+            continue  # saved at the head of the statement and restored by every instruction that changes it
+        if dest not in clobbers and dest not in out_sregs:
+            raise SystemExit(f"{what}: '{i['text']}' writes {dest}, which is neither an output nor a clobber")
+        # instructions that set SCC as a side effect
+        if re.match(r"s_(add|sub|addc|and|or)", parts[0]) and "scc" not in clobbers:
+            raise SystemExit(f"{what}: '{i['text']}' sets SCC, which is not a clobber")
+    execs = [i["text"] for i in ins if i["text"].startswith("s_mov_b64 exec")]
+    saves = [i["text"] for i in ins if i["text"] == "s_mov_b64 %[execsave], exec"]
+    if execs and (not saves or any("%[klast]" not in t and "%[vlast]" not in t and "%[execsave]" not in t for t in execs)):
+        raise SystemExit(f"{what}: EXEC is changed without being saved and restored")
+
+
 def operand_lists(c: Config):
     outs, ins, clob = [], [], []
     for db in range(c.DB):
@@ -528,7 +586,7 @@ def operand_lists(c: Config):
         outs.append((n, f"+{{s[{PTR_SGPR[n]}:{PTR_SGPR[n] + 1}]}}"))
     if c.elem == "f16":
         outs.append(("over", "+s"))
-    for n in ("tfill", "tnext", "tm0", "ringend", "klast", "vlast"):
+    for n in TEMP_SGPRS:
         outs.append((n, "=&s"))
     nq = 4 * c.NS
     for i in range(0, nq, 16):
@@ -556,18 +614,20 @@ def operand_lists(c: Config):
 def emit_macro(c: Config, out):
     ins = gen_loop(c)
     outs, inputs, clob = operand_lists(c)
-    temps = ("tfill", "tnext", "tm0", "ringend", "klast", "vlast")
+    check_clobbers(ins, outs, clob + SPECIAL_CLOBBERS, c.name)
+    temps = TEMP_SGPRS
     names = [n for n, _ in outs if n not in temps] + [n for n, _ in inputs]
     out.write(f"// {c.name}: {c.elem} D={c.D}, {c.NW} waves, {c.NSTG} stages; {c.nvgpr} vector registers\n")
     out.write(f"#define {c.name}_VGPRS {c.nvgpr}\n")
     out.write(f"#define {c.name}({', '.join('A_' + n for n in names)}) \\\n")
-    out.write("    do { unsigned t_fill_, t_next_, t_m0_, t_end_; unsigned long long t_kl_, t_vl_; asm volatile( \\\n")
+    out.write("    do { unsigned t_fill_, t_next_, t_m0_, t_end_; unsigned long long t_kl_, t_vl_, t_ex_; asm volatile( \\\n")
     for i in ins:
         out.write(f'        "{i["text"]}\\n\\t" \\\n')
-    tmpmap = {"tfill": "t_fill_", "tnext": "t_next_", "tm0": "t_m0_", "ringend": "t_end_", "klast": "t_kl_", "vlast": "t_vl_"}
+    tmpmap = {"tfill": "t_fill_", "tnext": "t_next_", "tm0": "t_m0_", "ringend": "t_end_", "klast": "t_kl_", "vlast": "t_vl_",
+              "execsave": "t_ex_"}
     o_s = ", ".join(f'[{n}] "{cs}"({tmpmap.get(n, "A_" + n)})' for n, cs in outs)
     i_s = ", ".join(f'[{n}] "{cs}"(A_{n})' for n, cs in inputs)
-    c_s = ", ".join(f'"{x}"' for x in ["memory", "vcc", "scc"] + clob)
+    c_s = ", ".join(f'"{x}"' for x in ["memory"] + SPECIAL_CLOBBERS + clob)
     out.write(f"        : {o_s} \\\n        : {i_s} \\\n        : {c_s}); }} while (0)\n\n")
 
 

@@ -144,7 +144,9 @@ int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTens
  * CHILL_BWD_NOALLOC_MAX_ROWS floats (16 MiB) that every GPU the library runs on holds until the process
  * ends; B * H * T beyond that returns CHILL_ERR_TOO_LARGE.  The call allocates and frees nothing.  All
  * calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race on
- * it; calls on one stream are ordered and need nothing more. */
+ * it; calls on one stream are ordered and need nothing more.  The FIRST call on a device looks the
+ * array's address up (hipGetSymbolAddress, under a lock), which may load the code object: make that call
+ * outside any stream capture; every later call on that device only launches kernels and may be captured. */
 #define CHILL_BWD_NOALLOC_MAX_ROWS (4 * 1024 * 1024)
 int chill_bwd_noalloc(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
                       const ChillTensor4* o, const ChillTensor4* d_o,

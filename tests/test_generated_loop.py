@@ -63,3 +63,27 @@ def test_check_catches_a_vector_write_right_before_its_mfma():
     with pytest.raises(SystemExit, match="too soon after a VALU write"):
         gen.check_stream(_stream(write, mfma), "no wait states")
     gen.check_stream(_stream(write, ("nop", "s_nop 1", [], [], {"nops": 2}), mfma), "two wait states")
+
+
+@pytest.mark.parametrize("elem,D,waves,stages", CONFIGS)
+def test_statement_declares_everything_it_writes(elem, D, waves, stages):
+    """The clobber list and the output operands of the generated statement cover every register its
+    instructions write (M0, VCC and SCC among them), and EXEC is saved and restored."""
+    c = gen.Config(elem, D, waves, stages)
+    ins = gen.gen_loop(c)
+    outs, inputs, clob = gen.operand_lists(c)
+    gen.check_clobbers(ins, outs, clob + gen.SPECIAL_CLOBBERS, c.name)
+    assert "m0" in gen.SPECIAL_CLOBBERS and any(i["text"].startswith("s_add_u32 m0") for i in ins)
+    # a list without M0, or without one of the scratch registers, is refused
+    with pytest.raises(SystemExit, match="writes m0"):
+        gen.check_clobbers(ins, outs, clob + ["vcc", "scc"], c.name)
+    with pytest.raises(SystemExit, match="neither an output nor a clobber"):
+        gen.check_clobbers(ins, outs, clob[1:] + gen.SPECIAL_CLOBBERS, c.name)
+    # so is a write to an input operand
+    bad = list(ins) + [dict(text="s_mov_b32 %[lds0], 0", kind="salu", reads=set(), writes=set(), nops=1, lds=False, wait=None)]
+    with pytest.raises(SystemExit, match="writes the input operand"):
+        gen.check_clobbers(bad, outs, clob + gen.SPECIAL_CLOBBERS, c.name)
+    # and an EXEC that is set without having been saved
+    unsaved = [i for i in ins if i["text"] != "s_mov_b64 %[execsave], exec"]
+    with pytest.raises(SystemExit, match="EXEC is changed"):
+        gen.check_clobbers(unsaved, outs, clob + gen.SPECIAL_CLOBBERS, c.name)

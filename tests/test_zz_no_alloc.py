@@ -73,6 +73,54 @@ def test_backward_without_workspace_equals_backward_with_one():
             assert torch.equal(got[name], want[name]), f"call {i}: {name} differs"
 
 
+def test_captured_in_a_hip_graph_after_a_first_call():
+    """chill_bwd_noalloc recorded into a HIP graph (its first call on the device has happened before, outside the
+    capture, as the header asks: that call looks the array's address up): every replay, with new contents in the
+    static inputs and eager work and synchronisations in between, equals the three entry points run eagerly."""
+    mask = ca.ChunkwiseChillMask(40, 1)
+    B, H, Hkv, T, D, dtype = 2, 4, 2, 300, 128, torch.bfloat16
+    backward_both_ways(mask, 1, 2, 2, 64, 64, dtype, None, seed=5)  # the first call on this device, if none was made yet
+    q, k, v, do = (torch.randn(B, h, T, D, device=DEV, dtype=dtype) for h in (H, Hkv, Hkv, H))
+    o = torch.empty_like(q)
+    lse = torch.empty(B, H, T, device=DEV)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    desc = mask.descriptor()
+    t = {n: _lib.tensor4(x) for n, x in (("q", q), ("k", k), ("v", v), ("o", o), ("do", do), ("dq", dq), ("dk", dk), ("dv", dv))}
+    r = lambda n: ctypes.byref(t[n])
+    L = _lib.lib
+    sm_scale = D ** -0.5
+
+    def forward(stream):
+        _lib.check("chill_fwd", L.chill_fwd(r("q"), r("k"), r("v"), r("o"), ctypes.c_void_p(lse.data_ptr()), _lib.strides3(lse), None, 0,
+                                            B, H, Hkv, T, D, _lib.BF16, sm_scale, ctypes.byref(desc), stream))
+
+    def backward(stream):
+        _lib.check("chill_bwd_noalloc", L.chill_bwd_noalloc(
+            r("q"), r("k"), r("v"), r("o"), r("do"), r("dq"), r("dk"), r("dv"), ctypes.c_void_p(lse.data_ptr()), _lib.strides3(lse),
+            None, 0, B, H, Hkv, T, D, _lib.BF16, sm_scale, ctypes.byref(desc), stream))
+
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        forward(stream)
+        backward(stream)
+    for replay in range(4):
+        for x in (q, k, v, do):
+            x.copy_(torch.randn_like(x) * (1.0 + 0.5 * replay))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [x.clone() for x in (dq, dk, dv)]
+        # eagerly, with a delta buffer of the caller, through the public operator's own backward
+        qe, ke, ve = (x.clone().requires_grad_() for x in (q, k, v))
+        out = ca.chill_attention(qe, ke, ve, mask=mask)
+        want = torch.autograd.grad(out, (qe, ke, ve), do)
+        torch.cuda.synchronize()
+        assert torch.equal(out, o), f"replay {replay}: forward"
+        for name, g, w in zip(("dq", "dk", "dv"), got, want):
+            assert torch.equal(g, w), f"replay {replay}: {name}"
+
+
 def test_sizes_beyond_the_array_are_refused():
     mask = ca.CausalChillMask()
     desc = mask.descriptor()
