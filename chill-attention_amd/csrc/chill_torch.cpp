@@ -180,8 +180,7 @@ class Attention : public torch::autograd::Function<Attention> {
                                                   int64_t mask_id, std::vector<int64_t> mask_args, double sm_scale,
                                                   bool return_lse) {
         at::AutoDispatchBelowADInplaceOrView below;
-        // (nothing is saved, and no LSE computed for it, where autograd is switched off)
-        const bool needs_grad = at::GradMode::is_enabled() && (q.requires_grad() || k.requires_grad() || v.requires_grad());
+        const bool needs_grad = q.requires_grad() || k.requires_grad() || v.requires_grad();
         auto [o, lse] = forward_impl(q, k, v, lens, entry_points, mask_id, mask_args, sm_scale, return_lse || needs_grad);
         if (needs_grad) {
             ctx->save_for_backward({q, k, v, o, lse, lens.has_value() && lens->defined() ? *lens : at::Tensor()});
@@ -209,6 +208,12 @@ std::tuple<at::Tensor, at::Tensor> attention_autograd(const at::Tensor& q, const
                                                       const c10::optional<at::Tensor>& lens, int64_t entry_points,
                                                       int64_t mask_id, at::IntArrayRef mask_args, double sm_scale,
                                                       bool return_lse) {
+    // where autograd is switched off (torch.no_grad) nothing is recorded: no LSE is computed for a backward that
+    // cannot come, and nothing is saved
+    if (!at::GradMode::is_enabled() || !(q.requires_grad() || k.requires_grad() || v.requires_grad())) {
+        at::AutoDispatchBelowADInplaceOrView below;
+        return forward_impl(q, k, v, lens, entry_points, mask_id, mask_args, sm_scale, return_lse);
+    }
     auto out = Attention::apply(q, k, v, lens, entry_points, mask_id, mask_args.vec(), sm_scale, return_lse);
     return {out[0], out[1]};
 }
