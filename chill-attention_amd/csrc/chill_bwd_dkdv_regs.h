@@ -28,8 +28,18 @@
 #include "chill_device.h"
 #include "chill_params.h"
 #include "chill_tiles.h"
+#include "chill_bwd_loop.inc"
 
 namespace chill {
+
+// Shapes whose runs of predicate-free tiles go through the generated loop (gen_bwd_loop.py).  Such a kernel
+// keeps V NEGATED in LDS: the dP chain of a block starts from delta and ends as dP' = delta - dO V^T, so that
+// dS' = P dP' = -dS costs one multiplication per entry, and dK^T is accumulated with the opposite sign and
+// stored times -sm_scale.
+template <typename E, int D, int CB, int NS>
+constexpr bool dkdv_has_generated_loop() {
+    return Elem<E>::k16 && D == 128 && CB == 2 && NS == 4;
+}
 
 template <typename E, int D, int MASK, int CB, int NS>
 __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_tiles, int total_items,
@@ -120,10 +130,25 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
     for (int i = 0; i <= LA; i++)
         if (i < n_iters) issue_iter(i, i);
 
+    constexpr bool kGen = dkdv_has_generated_loop<E, D, CB, NS>();
     const ET* kptr = reinterpret_cast<const ET*>(p.k) + b * p.sk.b + hkv * p.sk.h;
     const int kw = kb0 + KPW * wave;
     OperandOffsets<E, D> ofs;
     ofs.init(lane);
+    if constexpr (kGen) {
+        // every lane flips the sign of the V chunks it has loaded itself, once they are there (the first barrier
+        // of the loop stands between this and the first read of V)
+        wait_async_tiles();
+        constexpr int PER = TKR * L::CH / NT;
+#pragma unroll
+        for (int i = 0; i < PER; i++) {
+            i32x4* at = reinterpret_cast<i32x4*>(smem) + (i * NW + wave) * 64 + lane;
+            i32x4 x = *at;
+#pragma unroll
+            for (int e = 0; e < 4; e++) x[e] ^= (int)0x80008000;
+            *at = x;
+        }
+    }
     Resident<E, D> kf[CB];
 #pragma unroll
     for (int c = 0; c < CB; c++)
@@ -149,10 +174,83 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
 #pragma unroll
         for (int j = 0; j < NJ; j++) asm volatile("" ::"v"(kf[c].c[j]));
 
+    // What the generated loop takes besides K: per-lane LDS addresses with everything wave-dependent folded in
+    // (an LDS read of the loop is one of these registers plus a constant), the per-lane offsets of the tile
+    // loads, and scalars.
+    [[maybe_unused]] unsigned a_qrow[NJ], a_qtr[DB][2], a_vrow[NJ], a_vec = 0;
+    if constexpr (kGen) {
+        static_assert(L::kBlockAffine && OperandOffsets<E, D>::kHalfAffine, "rows of 256 bytes");
+        const unsigned ring = lds_address(smem + V_BYTES), vtile = lds_address(smem) + CB * wave * L::BLOCK_BYTES;
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            a_qrow[j] = ring + ofs.row[j];
+            a_vrow[j] = vtile + ofs.row[j];
+        }
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int w = 0; w < 2; w++) a_qtr[db][w] = ring + ofs.tr[db][0][w];
+        a_vec = ring + 2 * TILE_BYTES + 16 * h;
+    }
+    // first tile of iteration `it` and its pointers (the generated loop moves them on by itself)
+    auto tile_pointers = [&](int it, const ET*& qp, const ET*& dop, const float*& lsep, const float*& delp) {
+        const int g = it / n_tiles;
+        const int q0 = (wg.start + it % n_tiles) * TQS;
+        const int hq = hkv * p.group + g;
+        qp = reinterpret_cast<const ET*>(p.q) + b * p.sq.b + hq * p.sq.h + (int64_t)q0 * p.sq.t;
+        dop = reinterpret_cast<const ET*>(p.d_o) + b * p.sdo.b + hq * p.sdo.h + (int64_t)q0 * p.sdo.t;
+        lsep = p.lse + b * p.lse_b + hq * p.lse_h + q0;
+        delp = p.delta + b * p.delta_b + hq * p.delta_h + q0;
+    };
+    // Iterations [it, it + n) that the generated loop may run for this wave: the wave's tiles are predicate-free,
+    // and the tiles issued meanwhile (three ahead each) lie in the same query head and exist in full.
+    const int run_first = imax(ta, fa);
+    const int run_end = imin(imin(tb, fb), imin(n_tiles - (LA + 1), p.T / TQS - wg.start - (LA + 1)));
+
     int st_cur = NS - 1;
     int st_issue = LA;
     int tile = -1;  // position of iteration `it` inside the q-tile range (it % n_tiles)
     for (int it = 0; it < n_iters; it++) {
+        if constexpr (kGen) {
+            const int t_next = tile + 1 == n_tiles ? 0 : tile + 1;
+            int cnt = (t_next >= run_first) ? run_end - t_next : 0;
+            if (cnt >= 2 && p.scale_log2 != 0.f) {
+                const ET *qp, *dop;
+                const float *lsep, *delp;
+                tile_pointers(it + LA + 1, qp, dop, lsep, delp);
+                qp = uniform(qp), dop = uniform(dop), lsep = uniform(lsep), delp = uniform(delp);
+                cnt = uniform(cnt);
+                const int n_run = cnt;
+                const unsigned st0 = uniform((unsigned)(st_cur + 1 == NS ? 0 : st_cur + 1));
+                const unsigned ring = lds_address(smem + V_BYTES);
+                const unsigned dmabase = uniform(ring + wave * 1024), vecdma = uniform(ring + 2 * TILE_BYTES);
+                const unsigned qstep = uniform((unsigned)(TQS * p.sq.t * Elem<E>::kBytes));
+                const unsigned dostep = uniform((unsigned)(TQS * p.sdo.t * Elem<E>::kBytes));
+                const unsigned vecwave = uniform(wave == NW - 1 ? 1u : 0u);
+                const unsigned lane4 = lane * 4;
+                const float scale_s = uniform(p.scale_log2);
+#define CHILL_DKDV_LOOP_ARGS                                                                                          \
+    cnt, tok, qp, dop, lsep, delp, kf[0].c[0], kf[0].c[1], kf[0].c[2], kf[0].c[3], kf[0].c[4], kf[0].c[5], kf[0].c[6], \
+        kf[0].c[7], kf[1].c[0], kf[1].c[1], kf[1].c[2], kf[1].c[3], kf[1].c[4], kf[1].c[5], kf[1].c[6], kf[1].c[7],     \
+        a_qrow[0], a_qrow[1], a_qrow[2], a_qrow[3], a_qrow[4], a_qrow[5], a_qrow[6], a_qrow[7], a_qtr[0][0],            \
+        a_qtr[0][1], a_qtr[1][0], a_qtr[1][1], a_qtr[2][0], a_qtr[2][1], a_qtr[3][0], a_qtr[3][1], a_vrow[0],           \
+        a_vrow[1], a_vrow[2], a_vrow[3], a_vrow[4], a_vrow[5], a_vrow[6], a_vrow[7], a_vec, load_q.goff[0],             \
+        load_q.goff[1], load_do.goff[0], load_do.goff[1], lane4, scale_s, dmabase, vecdma, qstep, dostep, vecwave, st0
+#define CHILL_DKDV_LOOP_CALL(loop, ...) loop(__VA_ARGS__)
+                if constexpr (std::is_same<E, bf16_t>::value) {
+                    CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_BF16_128, CHILL_DKDV_LOOP_ARGS);
+                } else {
+                    CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_F16_128, CHILL_DKDV_LOOP_ARGS);
+                }
+#undef CHILL_DKDV_LOOP_CALL
+#undef CHILL_DKDV_LOOP_ARGS
+                st_cur = (st_cur + n_run) % NS;
+                st_issue = (st_issue + n_run) % NS;
+                tile = t_next + n_run - 1;
+                it += n_run - 1;
+                continue;
+            }
+        }
         wait_async_tiles();
         __syncthreads();
         st_cur = st_cur + 1 == NS ? 0 : st_cur + 1;
@@ -239,10 +337,12 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
                 });
             });
         }
+        // dS = P (dP - delta); with V negated the chain has delivered -dP, and dS' = P (delta - dP) = -dS
 #pragma unroll
         for (int c = 0; c < CB; c++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) dp[c][r] = s[c][r] * (dp[c][r] - del4[r / 4][r % 4]);
+            for (int r = 0; r < 16; r++)
+                dp[c][r] = kGen ? s[c][r] * (dp[c][r] + del4[r / 4][r % 4]) : s[c][r] * (dp[c][r] - del4[r / 4][r % 4]);
         // dK^T += Q^T dS
         {
             i32x4 sb[CB][2];
@@ -263,7 +363,8 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
         f32x16 acc[DB];
         const bool valid = k_pos < seq_len;
         static_for<DB>([&](auto db) { acc[db] = agpr_read_block<DK_BASE + 16 * (c * DB + db)>(); });
-        if (k_pos < p.T) store_row_transposed<E, D>(dkbase + (int64_t)k_pos * p.sdk.t, acc, p.sm_scale, valid, h);
+        if (k_pos < p.T)
+            store_row_transposed<E, D>(dkbase + (int64_t)k_pos * p.sdk.t, acc, kGen ? -p.sm_scale : p.sm_scale, valid, h);
         static_for<DB>([&](auto db) { acc[db] = agpr_read_block<DV_BASE + 16 * (c * DB + db)>(); });
         if (k_pos < p.T) store_row_transposed<E, D>(dvbase + (int64_t)k_pos * p.sdv.t, acc, 1.f, valid, h);
     });

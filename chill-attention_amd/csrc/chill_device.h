@@ -115,6 +115,20 @@ struct Elem<f32_t> {
     __device__ __forceinline__ static float to_float(type x) { return x; }
 };
 
+// A value that is the same in every lane, in a scalar register (says so where the compiler has lost track:
+// an "s" operand of an inline-asm statement must be one).
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ unsigned uniform(unsigned x) { return (unsigned)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ float uniform(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+}
+template <typename T>
+__device__ __forceinline__ const T* uniform(const T* p) {
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = uniform((unsigned)v), hi = uniform((unsigned)(v >> 32));
+    return (const T*)(((unsigned long long)hi << 32) | lo);
+}
+
 // Exchange a value between lane l and lane l ^ 32 (v_permlane32_swap).
 __device__ __forceinline__ float swap32(float x) {
     int xi = __builtin_bit_cast(int, x);

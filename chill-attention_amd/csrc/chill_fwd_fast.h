@@ -62,8 +62,6 @@ __device__ __forceinline__ i32x4 scale_chunk(i32x4 c, float f) {
     return Elem<E>::pack8(x);
 }
 
-__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
-__device__ __forceinline__ unsigned uniform(unsigned x) { return (unsigned)__builtin_amdgcn_readfirstlane((int)x); }
 
 // true if `mine` is true for any wave of the workgroup; flags = one int per wave in LDS
 template <int NW>
