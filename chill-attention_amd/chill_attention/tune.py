@@ -96,19 +96,22 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
 
 
 def check_hand_managed_registers(macros: dict | None = None) -> None:
-    """Raise RuntimeError unless, in every kernel that names accumulation registers itself (16-bit inputs,
-    head dim 256), the compiler stays below the registers the kernel names and spills nothing.  The check
-    reads the assembly hipcc writes for the given build (``macros`` as for the library build); it covers
-    register overlap and spills, nothing else.  Part of every build of the library."""
+    """Raise RuntimeError unless, in every kernel that names accumulation registers itself (16-bit inputs:
+    the three kernels of head dim 256, dK/dV with register-resident K at head dim 128), the compiler stays
+    below the registers the kernel names.  Spilled registers are accepted only where the compiler touches
+    no accumulation register at all (they are in scratch memory then, not parked in accumulation
+    registers).  The check reads the assembly hipcc writes for the given build (``macros`` as for the
+    library build); it covers register overlap and spills, nothing else.  Part of every build of the library."""
     for elem in ("bf16", "f16"):
-        rows = hand_managed_registers(elem, 256, macros)
-        if not rows:
-            raise RuntimeError(f"no hand-managed kernel found for {elem} head dim 256")
-        for name, compiler_max, hand_min, spilled in rows:
-            if compiler_max >= hand_min or spilled:
-                raise RuntimeError(
-                    f"kernel {name}: the compiler uses accumulation registers up to a{compiler_max} (the kernel "
-                    f"manages a{hand_min} and above itself) or spills ({spilled} registers): this build is unsound")
+        for dim in (256, 128):
+            rows = hand_managed_registers(elem, dim, macros)
+            if not rows:
+                raise RuntimeError(f"no hand-managed kernel found for {elem} head dim {dim}")
+            for name, compiler_max, hand_min, spilled in rows:
+                if compiler_max >= hand_min or (spilled and compiler_max >= 0):
+                    raise RuntimeError(
+                        f"kernel {name}: the compiler uses accumulation registers up to a{compiler_max} (the kernel "
+                        f"manages a{hand_min} and above itself) or spills ({spilled} registers): this build is unsound")
 
 
 def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | None = None) -> list:

@@ -1309,11 +1309,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(D >= 25
     }
 }
 
-// One (mask, tile shape): SMALL selects the table row for grids that would not fill the chip.
-template <typename E, int D, int MASK_ID, bool SMALL>
+// One (mask, tile shape): SMALL selects the table row for grids that would not fill the chip, REGS the one of
+// dkdv_regs_kernel where the shape has both kernels.
+template <typename E, int D, int MASK_ID, bool SMALL, bool REGS = false>
 int launch_dkdv_shape(const BwdParams& p, hipStream_t stream) {
-    constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, SMALL);
-    constexpr int CB = dkdv_regs_blocks(D, Elem<E>::kDType);
+    constexpr TileConfig cfg = dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, SMALL, REGS);
+    constexpr int CB = (REGS && dkdv_regs_is_optional(D, Elem<E>::kDType)) ? kDkdvRegsBlocks128 : dkdv_regs_blocks(D, Elem<E>::kDType);
     constexpr bool paired = dkdv_is_paired(D, Elem<E>::kDType) && CB == 0;
     static_assert(CB > 0 ? (cfg.rows == 128 * CB && cfg.streamed == 32 && cfg.waves == 4)
                          : paired ? (cfg.rows * 2 == cfg.waves * 32 && cfg.streamed == 64)
@@ -1357,8 +1358,12 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
         bool small = false;
         constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DKDV);
         if constexpr (served) small = bwd_takes_small((long long)p.B * p.H_kv, p.T, D, Elem<E>::kDType, CHILL_PASS_DKDV);
+        bool regs = false;
+        if constexpr (dkdv_regs_is_optional(D, Elem<E>::kDType)) regs = dkdv_takes_regs(MASK_ID, (long long)p.B * p.H_kv, p.T);
         if (small) {
             if constexpr (served) status = launch_bwd_small<E, D, MASK_ID, 2>(p, stream);
+        } else if (regs) {
+            if constexpr (dkdv_regs_is_optional(D, Elem<E>::kDType)) status = launch_dkdv_shape<E, D, MASK_ID, false, true>(p, stream);
         } else if constexpr (has_small_row) {
             status = dkdv_takes_small_row((long long)p.B * p.H_kv, p.T) ? launch_dkdv_shape<E, D, MASK_ID, true>(p, stream)
                                                                         : launch_dkdv_shape<E, D, MASK_ID, false>(p, stream);

@@ -261,11 +261,29 @@ constexpr int dkdv_regs_blocks(int D, int dtype) {
     return 0;
 }
 constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
+// 16-bit inputs at head dim 128 have both kernels: the paired one, and dkdv_regs_kernel with two blocks per wave,
+// whose runs of predicate-free tiles go through a generated loop (gen_bwd_loop.py).  The latter owns its CU (130 KiB of
+// LDS, 512 registers per wave) and pays more before and after its loop (K into registers, V negated in LDS, no second
+// workgroup to hide behind): it is taken for long sequences on a grid of at least two workgroups per CU, and not
+// for the banded masks, whose runs are a few tiles long.  Measured on dK/dV alone, against the paired kernel:
+// causal B8 H16 T8192 3.63 / 4.06 ms, B16 H16 T4096 2.18 / 2.27, B2 H8 T8192 0.547 / 0.591, full mask fp16 B4 H16
+// T4096 0.98 / 1.16, prefix-LM B4 H16 T8192 1.91 / 2.16; but causal B1 H8 T8192 0.368 / 0.318, B4 H16 T2048
+// 0.227 / 0.197, sliding window 512 at T8192 0.65 / 0.49; chunkwise (128, 2) fp16 B2 H32 T16384 0.74 / 0.75.
+constexpr int kDkdvRegsBlocks128 = 2;
+constexpr int kDkdvRegsMinSequence = 4096;
+constexpr int kDkdvRegsMinWorkgroups = 2 * 256;
+constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && D == 128 && !CHILL_TUNE_DKDV_R64; }
+constexpr bool dkdv_takes_regs(int mask_id, long long batch_kv_heads, int T) {
+    return !mask_is_banded(mask_id) && T >= kDkdvRegsMinSequence &&
+           batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >= kDkdvRegsMinWorkgroups;
+}
 
-constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype, bool small_grid = false) {
+// `regs`: the row of dkdv_regs_kernel where that kernel is an option (dkdv_regs_is_optional)
+constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype, bool small_grid = false, bool regs = false) {
     const int row_bytes = D * elem_bytes(dtype);
-    if (dkdv_regs_blocks(D, dtype) > 0) {
-        const int rows = 4 * 32 * dkdv_regs_blocks(D, dtype);
+    const int blocks = (regs && dkdv_regs_is_optional(D, dtype)) ? kDkdvRegsBlocks128 : dkdv_regs_blocks(D, dtype);
+    if (blocks > 0) {
+        const int rows = 4 * 32 * blocks;
         return TileConfig{rows, 32, 4, rows * row_bytes + dkdv_regs_stages(D) * (2 * 32 * row_bytes + 2 * 32 * 4)};
     }
     if (dkdv_is_paired(D, dtype)) {
@@ -304,7 +322,9 @@ inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_
                 *out = TileConfig{32, 32, kFwdSmallWaves, bwd_small_lds_bytes(D, dtype, 2)};
                 return CHILL_OK;
             }
-            *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T));
+            // (the row of long sequences on a full chip: the generated loop where there is one)
+            *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T),
+                                    T == kLongSequence ? !mask_is_banded(mask_id) : dkdv_takes_regs(mask_id, batch_heads, T));
             return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }

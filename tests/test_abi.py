@@ -108,8 +108,8 @@ def test_tile_table():
             for D in (16, 32, 64, 128, 256):
                 for p in (_lib.PASS_FWD, _lib.PASS_DQ, _lib.PASS_DKDV):
                     c = tile_config(mask, D, dt, p)
-                    # one wave per 32 resident rows, or (dK/dV) two or four waves per 32 rows
-                    assert c["rows"] in (32 * c["waves"], 16 * c["waves"], 8 * c["waves"]) and c["streamed"] % 32 == 0
+                    # one wave per 32 resident rows, or (dK/dV) two or four waves per 32 rows, or one wave per 64
+                    assert c["rows"] in (64 * c["waves"], 32 * c["waves"], 16 * c["waves"], 8 * c["waves"]) and c["streamed"] % 32 == 0
                     assert 0 < c["lds_bytes"] <= 160 * 1024
     # fp32 rows of 512 bytes and more: the waves of a 32-key block split its state
     assert tile_config(ca.CausalChillMask(), 128, torch.float32, _lib.PASS_DKDV)["waves"] == 8
@@ -139,9 +139,18 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
     assert _lib.lib.chill_tile_config_for_shape(1, 128, _lib.BF16, 0, 1, 0, (ctypes.c_int32 * 4)()) == -8
     # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU
-    for D, rows, waves in ((64, 64, 4), (32, 64, 4), (128, 128, 8)):
+    for D, rows, waves in ((64, 64, 4), (32, 64, 4)):
         c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV)
         assert (c["rows"], c["waves"]) == (rows, waves), (D, c)
+    # dK/dV at 16-bit head dim 128: K in registers, two 32-key blocks per wave (256 key rows, 4 waves, 32-row tiles in
+    # four stages) for long sequences on a grid of two workgroups per CU, except under banded masks; else the paired kernel
+    regs = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 256 * 256 + 4 * (2 * 32 * 256 + 2 * 32 * 4)}
+    assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_DKDV) == regs
+    assert tile_config(causal, 128, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs
+    assert tile_config(causal, 128, torch.float16, _lib.PASS_DKDV, seq_len=4096, batch_heads=32) == regs
+    for mask, T, bh in ((causal, 4095, 128), (causal, 4096, 31), (window, 8192, 128), (window, None, 1 << 20)):
+        c = tile_config(mask, 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
+        assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
     assert 2 * tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV)["lds_bytes"] <= 160 * 1024
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
     assert tq == 32 * waves and tk % 32 == 0
@@ -241,6 +250,12 @@ def test_hand_managed_accumulation_registers(elem):
             if kernel in name:
                 assert compiler_max < hand_min, (name, compiler_max, hand_min)
                 assert hand_min == lowest and spilled == 0, (name, hand_min, spilled)
+    # dK/dV with register-resident K at head dim 128 (a0..a255 named by the kernel and its generated loop): the
+    # compiler touches no accumulation register there, so what it spills is in scratch memory
+    rows = tune.hand_managed_registers(elem, 128)
+    assert len(rows) == 5 and all("dkdv_regs_kernel" in name for name, *_ in rows)
+    for name, compiler_max, hand_min, spilled in rows:
+        assert compiler_max == -1 and hand_min == 0, (name, compiler_max, hand_min)
 
 
 def test_eager_operator_library_loads():

@@ -423,6 +423,47 @@ def test_reference_max_is_raised_along_the_keys(case):
             assert (err[seen] <= tight + 1e-4 * want_lse[seen].abs()).all(), err[seen].max()
 
 
+# dK/dV at 16-bit head dim 128 on long sequences and full grids: K in registers, runs of predicate-free tiles in the
+# generated loop (chill_bwd_dkdv_regs.h, gen_bwd_loop.py).  id, dtype, B, H, H_kv, T, mask, lens
+DKDV_REGS_CASES = [
+    ("causal", torch.bfloat16, 2, 16, 16, 4096, ("CausalChillMask", ()), None),
+    ("causal-gqa-lens-f16", torch.float16, 4, 16, 8, 4096, ("CausalChillMask", ()), (4096, 4000, 33, 2049)),
+    ("full-gqa-ragged", torch.bfloat16, 2, 32, 16, 4100, ("FullChillMask", ()), None),
+    ("full-lens-f16", torch.float16, 2, 16, 16, 4130, ("FullChillMask", ()), (4130, 3000)),
+    ("prefix-lm", torch.bfloat16, 2, 16, 16, 4096, ("PrefixLMChillMask", (1024,)), None),
+    ("prefix-lm-gqa-ragged", torch.float16, 1, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001,)),
+]
+
+
+@pytest.mark.parametrize("case", DKDV_REGS_CASES, ids=lambda c: c[0])
+def test_dkdv_with_resident_keys_and_generated_loop(case):
+    """The dK/dV kernel that keeps K in registers and runs its predicate-free tiles in a generated loop, on shapes the
+    launcher routes to it (asserted from the tile table): heads of a GQA group one after the other, lens, sequence
+    lengths that leave a ragged last tile, the first tiles of a key block under the mask (run by the ordinary code).
+    Same bar as the other backward tests (chill_bwd_dkdv.py:347-508 is what it must equal)."""
+    _, dtype, B, H, Hkv, T, m, lens = case
+    D = 128
+    mask = make_mask(m)
+    cfg = tile_config(mask, D, dtype, _lib.PASS_DKDV, seq_len=T, batch_heads=B * Hkv)
+    assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
+    torch.manual_seed(stable_seed(case[0]))
+    q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    dout = torch.randn(B, H, T, D, device=DEV, dtype=dtype)
+    out = ca.chill_attention(q, k, v, mask=mask, lens=lens_t)
+    out.backward(dout)
+    qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+    ref, res_mask = orc.reference_naive(m[0], m[1], qf, kf, vf, lens_t)
+    ref.backward(dout.float() * res_mask)
+    check_close(out.detach() * res_mask, ref.detach(), dtype, OUT_TOL[dtype], D, "O")
+    for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
+        check_close(got, want, dtype, GRAD_TOL[dtype], D, name)
+    # rows at and behind lens get no gradient
+    if lens is not None:
+        for b, n in enumerate(lens):
+            assert (k.grad[b, :, n:] == 0).all() and (v.grad[b, :, n:] == 0).all()
+
+
 def test_rows_without_keys():
     """A query whose keys are all masked (possible with lens cutting a window that only looks ahead)."""
     m = ("SlidingWindowChillMask", (0, 0))

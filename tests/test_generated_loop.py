@@ -13,6 +13,11 @@ _spec = importlib.util.spec_from_file_location(
 gen = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(gen)
 
+_spec_b = importlib.util.spec_from_file_location(
+    "gen_bwd_loop", os.path.join(ROOT, "chill-attention_amd", "csrc", "gen_bwd_loop.py"))
+genb = importlib.util.module_from_spec(_spec_b)
+_spec_b.loader.exec_module(genb)
+
 CONFIGS = [("bf16", 128, 8, 4), ("f16", 128, 8, 4), ("bf16", 64, 4, 3), ("f16", 64, 4, 3)]
 
 
@@ -87,3 +92,56 @@ def test_statement_declares_everything_it_writes(elem, D, waves, stages):
     unsaved = [i for i in ins if i["text"] != "s_mov_b64 %[execsave], exec"]
     with pytest.raises(SystemExit, match="EXEC is changed"):
         gen.check_clobbers(unsaved, outs, clob + gen.SPECIAL_CLOBBERS, c.name)
+
+
+@pytest.mark.parametrize("elem", ["bf16", "f16"])
+def test_backward_loop_generates_and_declares_what_it_writes(elem):
+    """The generated loop of the dK/dV kernel with register-resident K (csrc/gen_bwd_loop.py): every path through the
+    statement (prologue of each stage, its iteration, the next ones, the exit) passes the hazard check, the ring of
+    operand registers comes back to where it started after the four unrolled stages, every register it writes is an
+    output or a clobber, and an iteration holds the 64 MFMAs and the LDS reads it is meant to."""
+    c = genb.Config(elem)
+    ins = genb.gen_statement(c)  # raises SystemExit if a hazard rule is broken or the ring does not close
+    outs, inputs, clob = genb.operand_lists(c)
+    genb.check_clobbers(ins, outs, clob + genb.SPECIAL_CLOBBERS, c.name)
+    with pytest.raises(SystemExit, match="neither an output nor a clobber"):
+        genb.check_clobbers(ins, outs, [x for x in clob if x != "a17"] + genb.SPECIAL_CLOBBERS, c.name)
+    cycle, orders = genb.find_steady_state(c)
+    assert c.NSTG % len(cycle) == 0 and c.nvgpr + 64 + 32 <= 256  # its own registers, K, addresses
+    it = genb.SteadyIteration(c, cycle[0], orders[-1])
+    st = genb.Stream()
+    assert it.generate(st, 0) == cycle[1 % len(cycle)]
+    text = [i["text"] for i in st.ins]
+    mf = [t for t in text if t.startswith("v_mfma")]
+    assert len(mf) == 64 and all(elem in t for t in mf)
+    # 32 of them accumulate into the sixteen dV^T / dK^T blocks in accumulation registers, each block exactly twice
+    acc = [t.split()[1].rstrip(",") for t in mf if t.split()[1].startswith("a[")]
+    assert len(acc) == 32 and all(acc.count(a) == 2 for a in set(acc)) and len(set(acc)) == 16
+    # LDS: 8 Q + 8 dO + 16 V row chunks, 16 transposed operands of two reads each, LSE2 and twice delta of the next tile
+    assert sum(t.startswith("ds_read_b128") for t in text) == 8 + 8 + 16 + 4 + 8
+    assert sum(t.startswith("ds_read_b64_tr_b16") for t in text) == 32
+    # vector work: 32 exponentials, 32 + 32 multiply(-add)s, 32 packs; four tile loads (and the two of the vectors)
+    assert sum(t.startswith("v_exp_f32") for t in text) == 32 and sum(t.startswith("v_fma_f32") for t in text) == 32
+    assert sum(t.startswith("v_mul_f32") for t in text) == 32 and sum(t.startswith(c.cvt) for t in text) == 32
+    assert sum(t.startswith("global_load_lds_dwordx4") for t in text) == 4 and sum(t.startswith("global_load_lds_dword ") for t in text) == 2
+    # every prefetched operand of the next iteration comes from the next stage
+    nxt = [t for t in text if "offset:" in t and int(t.split("offset:")[1]) >= c.stage and "%[vrow" not in t]
+    assert len(nxt) == 4 + 8 + 8
+
+
+def test_backward_loop_check_catches_a_missing_wait():
+    """The same stream with one of its computed waits removed does not pass."""
+    c = genb.Config("bf16")
+    cycle, orders = genb.find_steady_state(c)
+    it = genb.SteadyIteration(c, cycle[0], orders[-1])
+    pro, st = genb.Stream(), genb.Stream()
+    sch = genb.Sched(pro)
+    for text, regs in it.reads_for_stage(0):
+        sch.read(text, None, regs)
+    it.generate(st, 0)
+    tail = [dict(text="s_waitcnt lgkmcnt(0)", kind="wait", reads=set(), writes=set(), nops=1, lds=False, wait=0)]
+    genb.check_stream(pro.ins + st.ins + tail, "as generated")
+    waits = [n for n, i in enumerate(st.ins) if i["kind"] == "wait" and i["wait"] is not None and i["wait"] < 15]
+    broken = st.ins[:waits[3]] + st.ins[waits[3] + 1:]
+    with pytest.raises(SystemExit, match="in flight"):
+        genb.check_stream(pro.ins + broken + tail, "a wait removed")
