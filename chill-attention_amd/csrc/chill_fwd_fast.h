@@ -7,11 +7,16 @@
 //   * a row takes ONE reference m0, the max over its first visible block(s), before the loop; the
 //     score MFMA chains start from an accumulator block filled with -m0, so the exponent minus the
 //     reference comes out of the matrix pipe and P = exp2(acc) costs one instruction per entry;
-//   * the reference is never raised inside the loop.  O and LSE2 do not depend on it beyond rounding
-//     as long as the sums stay inside the range of the types: a row whose sum of P ends outside
-//     [kLo, kHi], or (fp16) any block sum above 2^15, marks the q-tile, and the kernel runs such a
-//     q-tile again through fwd_q_tile, whose softmax follows the running max.  Scores that drift by
-//     more than ~60 (bf16) / ~15 (fp16) log2 units from a row's first block are what it takes;
+//   * the reference is raised only where a row asks for it.  O and LSE2 do not depend on it beyond
+//     rounding as long as the sums stay inside the range of the types, so nothing is compared or rescaled
+//     block by block: a wave tests one sum per block (fp16: the lane's sum of P over the block against
+//     2^15) or per tile (bf16: the row sum against 2^40), and if any of its rows is above, a rare
+//     out-of-line block raises the references to the largest exponent at hand and rescales O^T, the row
+//     sums and the scores in flight (gen_raise in gen_fwd_loop.py; the same in plain_step below).
+//     Scores that climb by more than ~15 (fp16) / ~40 (bf16) log2 units above a row's reference are what
+//     it takes.  A row whose sum still ends outside [kLo, kHi] (a jump of more than ~80 units inside one
+//     tile, a NaN) marks the q-tile, and the kernel runs such a q-tile again through fwd_q_tile, whose
+//     softmax follows the running max block by block;
 //   * a step (32 keys) is software-pipelined two deep: while the matrix pipe runs O^T += V^T P(g)^T
 //     and then S(g+2)^T, the vector ALU turns S(g+1) into P(g+1) and the LDS reads of the operands
 //     of the other phase are in flight, every MFMA followed by its share of each.
@@ -38,14 +43,14 @@ struct FastSoftmaxLimits;
 template <>
 struct FastSoftmaxLimits<bf16_t> {
     static constexpr float kLo = 0x1p-60f, kHi = 0x1p60f;
-    static constexpr bool kBlockLimit = false;
     static constexpr float kBlockHi = 0.f;
+    static constexpr float kRaiseAbove = 0x1p40f;   // a lane's sum over a block that has the reference raised
 };
 template <>
 struct FastSoftmaxLimits<f16_t> {
     static constexpr float kLo = 0x1p-6f, kHi = 0x1p60f;
-    static constexpr bool kBlockLimit = true;  // every P of a block stays below 65504
-    static constexpr float kBlockHi = 32768.f;
+    static constexpr float kBlockHi = 32768.f;      // every P of a block stays below 65504 while the lane's sum does
+    static constexpr float kRaiseAbove = kBlockHi;
 };
 
 // bytes behind the ring: one flag per wave for the workgroup's vote on running the q-tile again
@@ -213,7 +218,6 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
             for (int r = 0; r < 16; r++) o[i][r] = 0.f;
         float l_run = 0.f;   // this lane's share of the row sum
         float m0 = 0.f;      // the row's reference (log2 domain, scale included)
-        bool over = false;   // fp16: a block sum went above the limit
         const int q_pos = qw + n;
         const Range vis = visible_range<MASK, true>(q_pos, seq_len, p.margs);  // the keys this lane's row sees
 
@@ -270,17 +274,42 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
             v_read(vo, stage, kb);
             float psum = 0.f;
             i32x4 pb[2];
+            auto softmax_block = [&]() {
+                psum = 0.f;
 #pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) {
-                f32x8 ps;
+                for (int s2 = 0; s2 < 2; s2++) {
+                    f32x8 ps;
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    ps[e] = fast_exp2(sc[8 * s2 + e]);
-                    psum += ps[e];
+                    for (int e = 0; e < 8; e++) {
+                        ps[e] = fast_exp2(sc[8 * s2 + e]);
+                        psum += ps[e];
+                    }
+                    pb[s2] = Elem<E>::pack8(ps);
                 }
-                pb[s2] = Elem<E>::pack8(ps);
+            };
+            softmax_block();
+            // a block whose sum leaves the range of P's type (fp16), or that takes the row sum far up (bf16): the
+            // reference of the rows is raised to the largest exponent of the block, as the generated loop does
+            if (__builtin_amdgcn_ballot_w64(psum > Lim::kRaiseAbove) != 0) {
+                float mx = sc[0];
+#pragma unroll
+                for (int r = 1; r < 16; r++) mx = fmaxf(mx, sc[r]);
+                const float d = fmaxf(max_across_halves(mx), 0.f);
+                const float alpha = fast_exp2(-d);
+                m0 += d;
+                l_run *= alpha;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    mneg[r] = -m0;
+                    sc[r] -= d;
+                }
+                asm volatile("" : "+v"(mneg));
+#pragma unroll
+                for (int db = 0; db < DB; db++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) o[db][r] *= alpha;
+                softmax_block();
             }
-            if (Lim::kBlockLimit) over |= psum > Lim::kBlockHi;
             l_run += psum;
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++)
@@ -362,28 +391,29 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
                         q0[4 * j + e] = qf.c[j][e];
                         q1[4 * j + e] = qf.c[(NJ > 4 ? 4 : 0) + j][e];
                     }
-                unsigned long long over_mask = 0;
                 const float block_hi = Lim::kBlockHi;
                 constexpr bool kBf16 = std::is_same<E, bf16_t>::value;
                 static_assert(decltype(load_k)::PER_WAVE == 3 && decltype(load_v)::PER_WAVE == 3, "three loads per wave and tile");
                 if constexpr (D == 128 && kBf16) {
-                    CHILL_FWD_LOOP_BF16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, q0, q1, mneg, k_lane,
+                    CHILL_FWD_LOOP_BF16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, mneg, q0, q1, k_lane,
                                                 v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
                                                 load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave);
                 } else if constexpr (D == 128) {
-                    CHILL_FWD_LOOP_F16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, over_mask, q0, q1, mneg,
-                                               k_lane, v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
+                    CHILL_FWD_LOOP_F16_128_8_4(o[0], o[1], o[2], o[3], l_run, cnt, rem, cur, kb, vb, mneg, q0, q1, k_lane,
+                                               v_lane, load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0],
                                                load_v.goff[1], load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
                 } else if constexpr (kBf16) {
-                    CHILL_FWD_LOOP_BF16_64_4_3(o[0], o[1], l_run, cnt, rem, cur, kb, vb, q0, mneg, k_lane, v_lane,
+                    CHILL_FWD_LOOP_BF16_64_4_3(o[0], o[1], l_run, cnt, rem, cur, kb, vb, mneg, q0, k_lane, v_lane,
                                                load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0], load_v.goff[1],
                                                load_v.goff[2], lds_base, kstep, vstep, w1024, wave);
                 } else {
-                    CHILL_FWD_LOOP_F16_64_4_3(o[0], o[1], l_run, cnt, rem, cur, kb, vb, over_mask, q0, mneg, k_lane, v_lane,
+                    CHILL_FWD_LOOP_F16_64_4_3(o[0], o[1], l_run, cnt, rem, cur, kb, vb, mneg, q0, k_lane, v_lane,
                                               load_k.goff[0], load_k.goff[1], load_k.goff[2], load_v.goff[0], load_v.goff[1],
                                               load_v.goff[2], lds_base, kstep, vstep, w1024, wave, block_hi);
                 }
-                if (Lim::kBlockLimit) over |= ((over_mask >> lane) & 1) != 0;
+                // the loop raises the reference where a row asks for it: what it leaves in the chain start is the
+                // reference from here on
+                m0 = -mneg[0];
                 st_cur = (st_cur + (i_hi - i_lo - 1)) % NS;
                 i = i_hi;
             }
@@ -409,7 +439,7 @@ __device__ __forceinline__ void fwd_fast_q_tiles(const FwdParams& p, char* smem,
                 lse_base[q_pos] = valid ? (l_tot == 0.f ? -INFINITY : m0 + __log2f(l_tot)) : 0.f;
         }
         // a row that sees keys must end with a sum inside the range (a NaN fails the comparison too)
-        const bool bad = (vis.lo <= vis.hi) && (over || !(l_tot >= Lim::kLo && l_tot <= Lim::kHi));
+        const bool bad = (vis.lo <= vis.hi) && !(l_tot >= Lim::kLo && l_tot <= Lim::kHi);
         const bool again = __builtin_amdgcn_ballot_w64(bad) != 0;
         if (workgroup_any<NW>(again, smem + NS * Lds::STAGE_BYTES)) {
             // rare: give the ring to the kernel whose softmax follows the running max, then start over on

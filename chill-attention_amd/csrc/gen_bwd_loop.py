@@ -8,7 +8,8 @@ registers, its dK^T / dV^T accumulators (2 x 2 x D/32 blocks) in the accumulatio
 An ITERATION takes one 32-row tile of Q and dO, with the LSE2 and delta of its rows, from a ring of
 four LDS stages and runs 64 MFMAs (D = 128), reference chill_attention/chill_bwd_dkdv.py:362-403:
 
-    phase A  slots  0..15   S_c    = Q K_c^T                 (c = 0, 1: the wave's two key blocks)
+    phase A  slots  0..15   S_c    = Q K_c^T                 (c = 0, 1: the wave's two key blocks; S_0 first, so that
+                                                          its exponentials can start eight slots earlier)
     phase B  slots 16..31   dP'_c  = delta - dO V_c^T        (V is stored negated; the chain starts from delta)
     phase C  slots 32..47   dV_c^T += dO^T P_c               P = exp2(S * scale - LSE2)
     phase D  slots 48..63   dK'_c^T += Q^T dS'_c             dS' = P * dP' = -dS   (the caller scales by -sm_scale)
@@ -19,8 +20,15 @@ them.  Operands are read into a ring of register units as early as units are fre
 `s_waitcnt lgkmcnt` is computed from the order of the reads.  At the end of an iteration the first
 operands of the next one (its LSE2, delta and Q chunks) are already on their way.
 
-The statement runs `cnt` consecutive iterations of one wave, each: wait for the tile ahead, barrier, issue
-the tile three ahead into the stage that has just been freed, 64 slots.  The caller guarantees that every
+The statement runs `cnt` consecutive iterations of one wave, each: issue the tile three ahead into the stage
+that has just been freed, 64 slots; the wait for the tile ahead and the barrier of the next iteration stand in
+front of slot 56, where every read of the current tile has returned, so that the last MFMAs cover the barrier.
+
+Measured on the causal bf16 B8 H16 T8192 workload (timing builds with parts of the loop left out, --ablate):
+the kernel takes 3.55 ms; without the LDS reads of the loop 3.15, without its vector instructions 3.35, without
+both 3.04, without its MFMAs 2.13, with none of the three (barriers, waits and everything outside the loop remain)
+0.85 ms.  A lone wave per SIMD issues at most one instruction every four cycles: ~330 instructions per 64 MFMAs
+leave little room, so the generator spreads the vector work over as many slots as the data dependences allow.  The caller guarantees that every
 tile of the run is predicate-free for the wave, that the tiles it issues exist in full and belong to one
 query head (the pointers advance by a fixed step), and does everything else itself.
 """
@@ -36,12 +44,13 @@ from asm_stream import AGPR, Stream, check_clobbers, check_stream, rng, vr  # no
 # fixed scalar register pairs of the four tile pointers (their halves are added to separately)
 PTR_SGPR = {"q": 88, "do": 90, "lse": 92, "del": 94}
 LGKM_MAX = 15   # the counter of outstanding LDS operations has four bits
+ABLATE = set()  # timing experiments only (--ablate): parts of the loop left out; the results are wrong
 TEMP_SGPRS = ("execsave",)
 SPECIAL_CLOBBERS = ["vcc", "scc", "m0"]
 
 
 class Config:
-    def __init__(self, elem: str, D: int = 128, units: int = 10):
+    def __init__(self, elem: str, D: int = 128, units: int = 10, barrier_slot: int = 56, split_a: bool = True):
         assert elem in ("bf16", "f16") and D == 128
         self.elem, self.D = elem, D
         self.CB, self.NSTG, self.NW = 2, 4, 4
@@ -61,6 +70,8 @@ class Config:
         self.T = r; r += 4
         self.nvgpr = r
         self.slots = 8 * self.NJ          # 64
+        self.split_a = split_a
+        self.barrier_slot = barrier_slot  # the barrier of the next iteration stands in front of this slot's MFMA
         self.mfma = "v_mfma_f32_32x32x16_" + elem
         self.cvt = "v_cvt_pk_bf16_f32" if elem == "bf16" else "v_cvt_pk_f16_f32"
         self.name = f"CHILL_DKDV_LOOP_{elem.upper()}_{D}"
@@ -76,6 +87,15 @@ class Config:
 def areg(base, n):
     b = base - AGPR
     return f"a[{b}:{b + n - 1}]"
+
+
+class AblatingStream(Stream):
+    """Drops the MFMAs of a timing experiment."""
+
+    def add(self, text, kind, *a, **kw):
+        if kind == "mfma" and "mfma" in ABLATE:
+            return
+        super().add(text, kind, *a, **kw)
 
 
 class Sched:
@@ -106,6 +126,15 @@ class Sched:
         done = self.seq - n
         for r in [r for r, s in self.pending.items() if s <= done]:
             del self.pending[r]
+
+    def wait_upto(self, seq):
+        """All reads up to sequence number `seq` have returned."""
+        n = min(self.seq - seq, LGKM_MAX)
+        if any(s <= seq for s in self.pending.values()):
+            self.st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
+            done = self.seq - n
+            for r in [r for r, s in self.pending.items() if s <= done]:
+                del self.pending[r]
 
     def wait_all(self):
         self.st.add("s_waitcnt lgkmcnt(0)", "wait", wait=0)
@@ -212,7 +241,7 @@ class Iteration:
                             rng(c.DP[blk] + 4 * g, 4)))
         return out
 
-    def generate(self, st: Stream, s: int, with_dma=True, with_prefetch=True):
+    def generate(self, st: Stream, s: int, with_dma=True, with_prefetch=True, with_barrier=True):
         """Returns the ring units that hold the Q chunks of the next iteration."""
         c = self.c
         nxt, tgt = (s + 1) % c.NSTG, (s + 3) % c.NSTG
@@ -230,9 +259,16 @@ class Iteration:
 
         # ---- the MFMAs, slot by slot: (text pieces, operand keys)
         slots = []
-        for j in range(c.NJ):
+        if c.split_a:
+            # S_0 in full, then S_1: the exponentials of block 0 can start eight slots earlier (a Q chunk stays in
+            # its ring unit for both)
             for blk in range(c.CB):
-                slots.append(("A", j, blk))
+                for j in range(c.NJ):
+                    slots.append(("A", j, blk))
+        else:
+            for j in range(c.NJ):
+                for blk in range(c.CB):
+                    slots.append(("A", j, blk))
         for j in range(c.NJ):
             for blk in range(c.CB):
                 slots.append(("B", j, blk))
@@ -311,23 +347,33 @@ class Iteration:
         valu = [[] for _ in range(NS)]
 
         def place(ops, lo, hi):
+            if "valu" in ABLATE:
+                return
             for t, lst in enumerate(deal(ops, lo, hi, NS)):
                 valu[t] += lst
-        e_ops = []
-        for half in (range(0, 4), range(4, 8)):
-            for blk in range(c.CB):
-                e_ops += softmax_pairs(c, st, blk, half)
-        place(e_ops, E_LO, E_HI)
+        if c.split_a:
+            place(softmax_pairs(c, st, 0, range(0, 8)), 10, 23)
+            place(softmax_pairs(c, st, 1, range(0, 4)), 24, 31)
+            place(softmax_pairs(c, st, 1, range(4, 8)), 32, E_HI)
+        else:
+            e_ops = []
+            for half in (range(0, 4), range(4, 8)):
+                for blk in range(c.CB):
+                    e_ops += softmax_pairs(c, st, blk, half)
+            place(e_ops, E_LO, E_HI)
         place(product_ops(c, st, 0, range(0, 8)) + product_ops(c, st, 1, range(0, 8)), G0_LO, G0_HI)
         place(pack_ops(c, st, 0, range(0, 4)) + pack_ops(c, st, 1, range(0, 4)), P0_LO, P0_HI)
         place(product_ops(c, st, 0, range(8, 16)) + product_ops(c, st, 1, range(8, 16)), G1_LO, G1_HI)
         place(pack_ops(c, st, 0, range(4, 8)) + pack_ops(c, st, 1, range(4, 8)), P1_LO, P1_HI)
-        scalar = deal(dma_ops(c, st, tgt), 0, 15, NS) if with_dma else [[] for _ in range(NS)]
+        scalar = deal(dma_ops(c, st, tgt), 0, 15, NS) if with_dma and "dma" not in ABLATE else [[] for _ in range(NS)]
 
         next_q = {}
         READS_PER_SLOT = 3
         self.prefetch_order = []
+        last_tile_read = 0   # sequence number of the last read of this iteration's tile
         for t, sl in enumerate(slots):
+            if t == c.barrier_slot and with_barrier:
+                self.early_barrier(st, sch, s, queue, last_tile_read)
             # operands and the MFMA
             if sl[0] == "A":
                 _, j, blk = sl
@@ -366,7 +412,10 @@ class Iteration:
                     break
                 unit = free.pop(free.index(min(free))) if needs_unit else None
                 for text, regs in read_text(key, unit):
-                    sch.read(text, None, regs)
+                    if "lds" not in ABLATE:
+                        sch.read(text, None, regs)
+                if key[0] in ("do", "dot", "qt"):
+                    last_tile_read = sch.seq
                 if key[0] == "nq":
                     next_q[key[1]] = unit
                 elif needs_unit:
@@ -387,12 +436,28 @@ class Iteration:
                     op()
             for op in scalar[t]:
                 op()
+        if c.barrier_slot >= NS and with_barrier:
+            self.early_barrier(st, sch, s, queue, last_tile_read)
         assert not queue, f"reads left over: {queue}"
         self.pending_after = dict(sch.pending)
         return [next_q[j] for j in range(c.NJ)] if with_prefetch else None
 
     def carried_order(self, carried):
         return carried
+
+    def early_barrier(self, st, sch, s, queue, last_tile_read):
+        """The barrier of the NEXT iteration, early enough for the MFMAs behind it to cover its latency: every
+        read of this iteration's tile has returned (the stage is refilled after the barrier), and the tile two
+        ahead has landed.  The last iteration of a run leaves that barrier to the caller."""
+        c = self.c
+        assert not any(k[0] in ("do", "dot", "qt") for k, _ in queue), "reads of the tile behind the barrier"
+        sch.wait_upto(last_tile_read)
+        st.add("s_cmp_eq_u32 %[cnt], 1", "salu")
+        st.add(f"s_cbranch_scc1 .Lnobar{s}%=", "salu")
+        st.add(f"s_waitcnt vmcnt({c.loads_per_tile})", "wait")
+        if "barrier" not in ABLATE:
+            st.add("s_barrier", "salu")
+        st.add(f".Lnobar{s}%=:", "label", nops=0)
 
 
 def find_steady_state(c: Config):
@@ -463,15 +528,13 @@ def gen_statement(c: Config):
             sch.read(text, None, regs)
         pro.add(f"s_branch .Lbody{s}%=", "salu")
         pros.append(pro)
-        body = Stream()
+        body = AblatingStream()
         body.add(f".Lbody{s}%=:", "label", nops=0)
         nq = its[s].generate(body, s)
         assert nq == cycle[(s + 1) % n] and its[s].prefetch_order == orders[s % n]
         body.add("s_sub_u32 %[cnt], %[cnt], 1", "salu")
         body.add("s_cmp_eq_u32 %[cnt], 0", "salu")
         body.add("s_cbranch_scc1 .Lexit%=", "salu")
-        body.add(f"s_waitcnt vmcnt({c.loads_per_tile})", "wait")
-        body.add("s_barrier", "salu")
         if s == c.NSTG - 1:
             body.add("s_branch .Lbody0%=", "salu")
         bodies.append(body)
@@ -479,7 +542,7 @@ def gen_statement(c: Config):
     tail.add(".Lexit%=:", "label", nops=0)
     tail.add("s_waitcnt lgkmcnt(0)", "wait", wait=0)
     # the hazards of every path: a prologue, its body, the next body, the exit
-    for s in range(c.NSTG):
+    for s in range(c.NSTG if not ABLATE else 0):
         n = (s + 1) % c.NSTG
         check_stream(pros[s].ins + bodies[s].ins + bodies[n].ins + bodies[(n + 1) % c.NSTG].ins + tail.ins,
                      f"{c.name} (from stage {s})")
@@ -544,10 +607,19 @@ def emit_macro(c: Config, out):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("-o", "--output", default="chill_bwd_loop.inc")
+    ap.add_argument("--barrier-slot", type=int, default=None, help="timing experiments: slot of the early barrier")
+    ap.add_argument("--units", type=int, default=None, help="timing experiments: ring units")
+    ap.add_argument("--split-a", type=int, default=None, help="timing experiments: S_0 before S_1")
+    ap.add_argument("--ablate", default="", help="timing experiments: comma-separated parts to leave out "
+                                                 "(barrier, valu, lds, dma, mfma); the results are wrong")
     args = ap.parse_args()
+    ABLATE.update(x for x in args.ablate.split(",") if x)
     with open(args.output, "w") as out:
         out.write("// Generated by gen_bwd_loop.py; do not edit.\n#pragma once\n\n")
-        for c in (Config("bf16"), Config("f16")):
+        if ABLATE:
+            out.write("#ifndef CHILL_TIMING_EXPERIMENT\n#error \"a loop with parts left out (--ablate): timing experiments only\"\n#endif\n\n")
+        kw = {k: v for k, v in (("barrier_slot", args.barrier_slot), ("units", args.units), ("split_a", args.split_a)) if v is not None}
+        for c in (Config("bf16", **kw), Config("f16", **kw)):
             emit_macro(c, out)
     return 0
 

@@ -127,12 +127,73 @@ def softmax_ops(c: Config, st: Stream, s_in: int, p_out: int):
     return ops
 
 
-def block_sum_check(c: Config, st: Stream):
-    if c.elem == "f16" and "valu" not in c.ablate:
-        # every P of the block stays below 65504 while the block sum does; the flag is sticky
-        st.add(f"v_cmp_lt_f32 vcc, %[blockhi], {vr(c.PSUM)}", "valu", [c.PSUM], [])
-        st.add("s_or_b64 %[over], %[over], vcc", "salu")
+RAISE_ROW_SUM = "0x53800000"   # 2^40: a row sum above it has the reference raised (bf16; P and the sum reach 2^127)
+
+
+def block_sum_check(c: Config, st: Stream, par: int, tag: str, tile_end: bool = True):
+    """End of a step whose vector work has produced P[par ^ 1] from S[par ^ 1] (and, in the loop, whose matrix work
+    has left the scores after those in S[par]): the row sums, and the test that sends the wave to `gen_raise`.
+    fp16: every P of a block stays below 65504 while the lane's sum over the block stays below `blockhi`, tested after
+    every block; bf16: the row sum is tested once per tile.  The branch is taken by the whole wave if any row asks."""
+    if "valu" in c.ablate:
+        return
+    if c.elem == "f16":
         st.add(f"v_add_f32 {vr(c.L)}, {vr(c.L)}, {vr(c.PSUM)}", "valu", [c.L, c.PSUM], [c.L])
+        st.add(f"v_cmp_lt_f32 vcc, %[blockhi], {vr(c.PSUM)}", "valu", [c.PSUM], [])
+    elif tile_end:
+        st.add(f"v_cmp_lt_f32 vcc, {RAISE_ROW_SUM}, {vr(c.L)}", "valu", [c.L], [])
+    else:
+        return
+    st.ins.append(dict(text=f"s_cbranch_vccnz .Lraise{tag}%=", kind="raise", reads=set(), writes=set(), nops=1, lds=False,
+                       wait=None, par=par, tag=tag))
+    st.add(f".Lback{tag}%=:", "label", nops=0)
+
+
+def gen_raise(c: Config, st: Stream, par: int):
+    """The reference of the rows is raised by d = the largest exponent among the scores at hand (never lowered):
+    S[par ^ 1] (whose P is packed in P[par ^ 1] and not yet part of O^T) and S[par]; the scores at hand, the start
+    value of the score chains, O^T and the row sum follow, and P[par ^ 1] is computed again.  O^T and LSE2 do not
+    depend on the reference beyond rounding (the running max of chill_fwd.py:188-286 does the same, block by block).
+    Rare: the block is out of line."""
+    A = st.add
+    ripe, fresh, P = c.S[par ^ 1], c.S[par], c.P[par ^ 1]
+    d, t0, t1, t2 = c.PSUM, c.T, c.T + 1, c.T + 2
+    # what the matrix pipe may still be working on: the scores in `fresh`, O^T
+    A("s_nop 7", "nop", nops=8)
+    A("s_nop 7", "nop", nops=8)
+    regs = rng(ripe, 16) + rng(fresh, 16)
+    A(f"v_max3_f32 {vr(t0)}, {vr(regs[0])}, {vr(regs[1])}, {vr(regs[2])}", "valu", regs[:3], [t0])
+    rest = regs[3:]
+    while len(rest) >= 2:
+        A(f"v_max3_f32 {vr(t0)}, {vr(t0)}, {vr(rest[0])}, {vr(rest[1])}", "valu", [t0] + rest[:2], [t0])
+        rest = rest[2:]
+    if rest:
+        A(f"v_max_f32 {vr(t0)}, {vr(t0)}, {vr(rest[0])}", "valu", [t0, rest[0]], [t0])
+    # the two lanes of a row (l and l ^ 32) hold half of its keys each and share its reference
+    A(f"v_mov_b32 {vr(t1)}, {vr(t0)}", "valu", [t0], [t1])
+    A("s_nop 1", "nop", nops=2)
+    A(f"v_permlane32_swap_b32 {vr(t0)}, {vr(t1)}", "valu", [t0, t1], [t0, t1])
+    A(f"v_max_f32 {vr(d)}, {vr(t0)}, {vr(t1)}", "valu", [t0, t1], [d])
+    A(f"v_max_f32 {vr(d)}, 0, {vr(d)}", "valu", [d], [d])
+    for r in regs + rng(c.MNEG, 16):
+        A(f"v_sub_f32 {vr(r)}, {vr(r)}, {vr(d)}", "valu", [r, d], [r])
+    A(f"v_exp_f32 {vr(t2)}, -{vr(d)}", "trans", [d], [t2])
+    A("s_nop 0", "nop")
+    A(f"v_mul_f32 {vr(c.L)}, {vr(c.L)}, {vr(t2)}", "valu", [c.L, t2], [c.L])
+    for r in rng(c.O, 16 * c.DB):
+        A(f"v_mul_f32 {vr(r)}, {vr(r)}, {vr(t2)}", "valu", [r, t2], [r])
+    # P again, against the new reference (its share of the row sum has been scaled with the sum)
+    pend = None
+    for k in range(8):
+        ta, tb = c.T + (2 * k) % 4, c.T + (2 * k + 1) % 4
+        A(f"v_exp_f32 {vr(ta)}, {vr(ripe + 2 * k)}", "trans", [ripe + 2 * k], [ta])
+        A(f"v_exp_f32 {vr(tb)}, {vr(ripe + 2 * k + 1)}", "trans", [ripe + 2 * k + 1], [tb])
+        if pend is not None:
+            A(*pend[:2], pend[2], pend[3])
+        pend = (f"{c.cvt} {vr(P + k)}, {vr(ta)}, {vr(tb)}", "valu", [ta, tb], [P + k])
+    A("s_nop 0", "nop")
+    A(*pend[:2], pend[2], pend[3])
+    A("s_nop 1", "nop", nops=2)
 
 
 def mfma_pv(c: Config, st: Stream, t: int, p_in: int):
@@ -180,7 +241,7 @@ def wait_lgkm(st: Stream, n: int):
     st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
 
 
-def gen_step(c: Config, st: Stream, par: int, filler=(), late_filler=()):
+def gen_step(c: Config, st: Stream, par: int, filler=(), late_filler=(), tag=""):
     """One step.  `filler`: closures (scalar work: ring rotation, tile loads) dealt over all slots;
     `late_filler`: closures dealt over the slots of the second phase only."""
     NS = c.NS
@@ -216,7 +277,7 @@ def gen_step(c: Config, st: Stream, par: int, filler=(), late_filler=()):
         read_v(c, st, t, c.VA[par], par ^ 1)
         fill_slot(NS + t)
     assert next(it, None) is None and next(fit, None) is None and next(lit, None) is None
-    block_sum_check(c, st)
+    block_sum_check(c, st, par, tag + str(par), tile_end=(par == 1))
 
 
 def issue_ops(c: Config, st: Stream):
@@ -330,7 +391,7 @@ def gen_fill(c: Config, st: Stream):
     A("s_nop 7", "nop", nops=8)
     for op in softmax_ops(c, st, c.S[0], c.P[0]):
         op()
-    block_sum_check(c, st)
+    block_sum_check(c, st, 1, "fill")   # as after a step of parity 1: P[0] from S[0], newer scores in S[1]
     for t in range(c.NS):
         read_v(c, st, t, c.VA[0], 0)
 
@@ -349,7 +410,9 @@ def gen_drain(c: Config, st: Stream):
         read_v(c, st, t, c.VA[0], 1)
         for _ in range(share[t]):
             next(it)()
-    block_sum_check(c, st)
+    # as after a step of parity 0: P[1] from S[1]; S[0] holds scores the row has already taken in, which no
+    # reference needs to stay below
+    block_sum_check(c, st, 0, "drain")
     st.add("s_nop 1", "nop", nops=2)
     for t in range(NS):
         wait_lgkm(st, 2 * (NS - 1 - t))
@@ -396,25 +459,37 @@ def gen_loop(c: Config):
     gen_fill(c, fill)
     # fast tile: the pending loads under step 0, the rotation under step 1 (the K address of the next
     # tile behind the last K read of step 1), then only the wait and the barrier between tiles
-    gen_step(c, fast, 0, filler=issue_ops(c, fast))
-    gen_step(c, fast, 1, filler=rotate_ops(c, fast),
+    gen_step(c, fast, 0, filler=issue_ops(c, fast), tag="fast")
+    gen_step(c, fast, 1, filler=rotate_ops(c, fast), tag="fast",
              late_filler=[lambda: fast.add(f"v_add_u32 {vr(c.KA)}, %[tnext], {vr(c.KLANE)}", "valu", [c.KLANE], [c.KA])])
     fast.add(f"s_waitcnt vmcnt({c.FL * c.loads_min})", "wait")
     if "barrier" not in c.ablate:
         fast.add("s_barrier", "salu")
     fast.add(f"v_mov_b32 {vr(c.VA[0])}, {vr(c.VA[1])}", "valu", [c.VA[1]], [c.VA[0]])
     fast.add(f"v_add_u32 {vr(c.VA[1])}, %[tnext], {vr(c.VLANE)}", "valu", [c.VLANE], [c.VA[1]])
-    gen_step(c, steps, 0)
-    gen_step(c, steps, 1)
+    gen_step(c, steps, 0, tag="rest")
+    gen_step(c, steps, 1, tag="rest")
     gen_ring_top(c, top, "")
     gen_issue_now(c, pre_drain)
     gen_drain(c, drain)
-    # what can follow what
+    # what can follow what, with no reference raised and with every one of them raised
+    def raised(ins):
+        out = []
+        for i in ins:
+            out.append(i)
+            if i["kind"] == "raise":
+                body = S()
+                gen_raise(c, body, i["par"])
+                out += body.ins
+        return out
+
     if not c.ablate:
-        check_stream(head.ins + fill.ins + pre_drain.ins + drain.ins, c.name + " (one tile)")
-        check_stream(head.ins + fill.ins + fast.ins + fast.ins + fast.ins + pre_drain.ins + drain.ins, c.name + " (fast)")
-        check_stream(head.ins + fill.ins + fast.ins + fast.ins + steps.ins + top.ins + steps.ins + top.ins + drain.ins,
-                     c.name + " (fast, then the last tiles)")
+        for how, path in (("", lambda x: x), (", references raised", raised)):
+            check_stream(path(head.ins + fill.ins + pre_drain.ins + drain.ins), c.name + " (one tile)" + how)
+            check_stream(path(head.ins + fill.ins + fast.ins + fast.ins + fast.ins + pre_drain.ins + drain.ins),
+                         c.name + " (fast)" + how)
+            check_stream(path(head.ins + fill.ins + fast.ins + fast.ins + steps.ins + top.ins + steps.ins + top.ins + drain.ins),
+                         c.name + " (fast, then the last tiles)" + how)
     out = S()
     out.ins += head.ins + fill.ins
     # fast tiles while a load is pending and a tile follows
@@ -441,6 +516,15 @@ def gen_loop(c: Config):
     out.add("s_branch .Lrest%=", "salu")
     out.add(".Ldrain%=:", "label", nops=0)
     out.ins += drain.ins
+    # out of line: the blocks that raise the reference of the rows, one per place that may ask for it
+    places = [i for i in out.ins if i["kind"] == "raise"]
+    if places:
+        out.add("s_branch .Lend%=", "salu")
+        for i in places:
+            out.add(f".Lraise{i['tag']}%=:", "label", nops=0)
+            gen_raise(c, out, i["par"])
+            out.add(f"s_branch .Lback{i['tag']}%=", "salu")
+        out.add(".Lend%=:", "label", nops=0)
     return out.ins
 
 
@@ -458,15 +542,13 @@ def operand_lists(c: Config):
         outs.append((n, "+s"))
     for n in ("kb", "vb"):
         outs.append((n, f"+{{s[{PTR_SGPR[n]}:{PTR_SGPR[n] + 1}]}}"))
-    if c.elem == "f16":
-        outs.append(("over", "+s"))
+    outs.append(("mneg", f"+{{v[{c.MNEG}:{c.MNEG + 15}]}}"))
     for n in TEMP_SGPRS:
         outs.append((n, "=&s"))
     nq = 4 * c.NS
     for i in range(0, nq, 16):
         w = min(16, nq - i)
         ins.append((f"q{i // 16}", f"{{v[{c.Q + i}:{c.Q + i + w - 1}]}}"))
-    ins.append(("mneg", f"{{v[{c.MNEG}:{c.MNEG + 15}]}}"))
     ins.append(("klane", f"{{v{c.KLANE}}}"))
     ins.append(("vlane", f"{{v{c.VLANE}}}"))
     for j in range(c.kper):

@@ -326,6 +326,13 @@ RAMP_CASES = [
     ("d128-loop-paired-one-wave", torch.bfloat16, 128, 4, 16, 16, 2048, (256, 8), (0, 1, 7), "wave", None),
     ("d128-loop-paired-lens", torch.bfloat16, 128, 4, 16, 8, 2048, (256, 8), (0, 1, 7), "all", (2048, 1500, 300, 2047)),
     ("d128-loop-paired-lens-f16", torch.float16, 128, 4, 16, 16, 2048, (256, 8), (1,), "low", (700, 2048, 1, 1025)),
+    # "step": the scores jump by the whole growth at key T / 2 instead of climbing to it: more than a sum inside the
+    # loop can take within one tile, so these q-tiles are voted on and computed again by fwd_q_tile on the same LDS ring
+    ("d128-loop-paired-step", torch.bfloat16, 128, 4, 16, 16, 2048, (256, 8), (0, 1, 7), "step", None),
+    ("d128-loop-paired-step-f16", torch.float16, 128, 4, 16, 8, 2048, (256, 8), (0, 1), "step-low", (2048, 1500, 300, 2047)),
+    ("d128-loop-unpaired-step", torch.bfloat16, 128, 2, 8, 8, 2048, (256, 8), (0, 1), "step-wave", None),
+    ("d64-loop-step", torch.bfloat16, 64, 8, 16, 16, 2048, (128, 4), (0, 1, 7), "step-low", None),
+    ("d64-loop-step-f16", torch.float16, 64, 2, 8, 4, 1024, (128, 4), (0, 1), "step", None),
     ("d64-loop", torch.bfloat16, 64, 2, 8, 8, 1024, (128, 4), (0, 1, 4), "all", None),
     ("d64-loop-f16", torch.float16, 64, 2, 8, 4, 1024, (128, 4), (0, 1, 4), "all", None),
     ("d64-loop-paired-second-only", torch.float16, 64, 8, 16, 16, 2048, (128, 4), (0, 1, 7), "low", None),
@@ -347,17 +354,21 @@ RAMP_CASES = [
 # 2^21 implies for up to 64 blocks), and what the test feeds
 RAMP_TRIP = {torch.bfloat16: 60.0, torch.float16: 21.0, torch.float32: 0.0}
 RAMP_GROWTH = {torch.bfloat16: 400.0, torch.float16: 60.0, torch.float32: 60.0}
+STEP_GROWTH = {torch.bfloat16: 400.0, torch.float16: 300.0}
 
 
 @pytest.mark.parametrize("case", RAMP_CASES, ids=lambda c: c[0])
 def test_reference_max_is_raised_along_the_keys(case):
     """Scores that grow by RAMP_GROWTH (log2 units) along the key axis, for the rows selected by `drift`: the
     forward's reference max has to follow them.  Every forward kernel has its own way (running max; a guarded raise;
-    the reference-free softmax of the generated loops, whose q-tiles are then voted on and computed again by
-    fwd_q_tile): one case per kernel and way, with the route asserted from the tile table.  O and LSE2 against the
+    the softmax of the generated loops, which raises a row's reference only when a sum leaves a guarded range, in an
+    out-of-line block of the generated statement and in the steps around it): one case per kernel and way, with the
+    route asserted from the tile table.  O and LSE2 against the
     oracle (chill_fwd.py:188-286 is the running-max softmax all of them must equal)."""
     _, dtype, D, B, H, Hkv, T, route, mask_ix, drift, lens = case
-    growth = RAMP_GROWTH[dtype]
+    step = drift.startswith("step")
+    drift = {"step": "all", "step-low": "low", "step-wave": "wave"}.get(drift, drift)
+    growth = STEP_GROWTH[dtype] if step else RAMP_GROWTH[dtype]
     torch.manual_seed(7)
     q = torch.randn(B, H, T, D, device=DEV) * 0.5
     k = torch.randn(B, Hkv, T, D, device=DEV) * 0.5
@@ -371,6 +382,8 @@ def test_reference_max_is_raised_along_the_keys(case):
     q = q - (q @ u)[..., None] * u
     q = q + 4.0 * carries[None, None, :, None] * u
     ramp = torch.arange(T, device=DEV, dtype=torch.float32) / T
+    if step:
+        ramp = (ramp >= (0.25 if drift == "low" else 0.5)).float()
     k = k + (growth * (D ** 0.5) / (4.0 * 1.4427)) * ramp[None, None, :, None] * u
     q, k, v = (x.to(dtype) for x in (q, k, v))
     lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
@@ -409,15 +422,13 @@ def test_reference_max_is_raised_along_the_keys(case):
         if dtype != torch.float32 and D in (64, 128) and route != (32, 4) and not (D == 128 and route == (128, 4)):
             # The generated loops take Q already multiplied by scale * log2(e) and rounded to the input type (what the
             # reference's PRESCALE_QK does, chill_fwd.py:120-127, chill_bwd_dkdv.py:118): the exponent of a (query, key)
-            # pair then carries the rounding errors of D products, each up to eps * |q_d * k_d| * scale * log2(e): four
-            # standard deviations of their sum for independent roundings are allowed here.  (The keys of this test
-            # reach a norm of several hundred.)  Rows that leave the range are computed again from the unrounded Q
-            # and meet the tight bar.
+            # pair then carries the rounding errors of D products, each up to eps * |q_d * k_d| * scale * log2(e), in sum
+            # at most eps * |q| * |k| * scale * log2(e).  (The keys of this test reach a norm of several hundred: the
+            # bound is ~1.4 log2 units where LSE2 is ~400; the observed errors reach half of it.)
             eps = {torch.bfloat16: 2.0 ** -9, torch.float16: 2.0 ** -12}[dtype]
             k_norm = k.float().norm(dim=-1).amax(dim=-1)  # [B, H_kv]
             k_norm = k_norm.repeat_interleave(H // Hkv, dim=1)[..., None]
-            loose = 4.0 * eps * (D ** -0.5 * 1.4427) * q.float().norm(dim=-1) * k_norm / D ** 0.5
-            assert (err[seen & risen] <= tight + 1e-4 * want_lse[seen & risen].abs()).all(), err[seen & risen].max()
+            loose = eps * (D ** -0.5 * 1.4427) * q.float().norm(dim=-1) * k_norm
             assert (err[seen] <= (tight + loose)[seen]).all(), (err - loose)[seen].max()
         else:
             assert (err[seen] <= tight + 1e-4 * want_lse[seen].abs()).all(), err[seen].max()
