@@ -9,6 +9,7 @@ from __future__ import annotations
 
 AGPR = 1000             # register number of a0 in the bookkeeping
 
+LGKM_MAX = 15           # the counter of outstanding LDS operations has four bits
 MFMA_RESULT_WAIT = 11   # wait states before a non-MFMA instruction may read an 8-pass MFMA result
 VALU_TO_MFMA_WAIT = 2   # wait states between a VALU write and an MFMA that reads the register
 TRANS_USE_WAIT = 1      # wait states between v_exp_f32 and a VALU read of its result
@@ -152,3 +153,60 @@ def check_clobbers(ins, outs, clobbers, what):
             restored = t == "s_mov_b64 exec, %[execsave]"
     if not restored:
         raise SystemExit(f"{what}: EXEC is changed without being saved and restored")
+
+
+def areg(base, n):
+    b = base - AGPR
+    return f"a[{b}:{b + n - 1}]"
+
+
+class Sched:
+    """Emits into a Stream, keeps the order of the LDS reads and computes the waits."""
+
+    def __init__(self, st: Stream, carried=()):
+        self.st = st
+        self.seq = 0
+        self.pending = {}
+        for regs in carried:      # reads of the iteration before that may still be in flight, oldest first
+            self.seq += 1
+            for r in regs:
+                self.pending[r] = self.seq
+
+    def read(self, text, addr, regs):
+        self.st.add(text, "lds", [], regs, lds=True)
+        self.seq += 1
+        for r in regs:
+            self.pending[r] = self.seq
+
+    def need(self, regs):
+        seqs = [self.pending[r] for r in regs if r in self.pending]
+        if not seqs:
+            return
+        last = max(seqs)
+        n = min(self.seq - last, LGKM_MAX)
+        self.st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
+        done = self.seq - n
+        for r in [r for r, s in self.pending.items() if s <= done]:
+            del self.pending[r]
+
+    def wait_upto(self, seq):
+        """All reads up to sequence number `seq` have returned."""
+        n = min(self.seq - seq, LGKM_MAX)
+        if any(s <= seq for s in self.pending.values()):
+            self.st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
+            done = self.seq - n
+            for r in [r for r, s in self.pending.items() if s <= done]:
+                del self.pending[r]
+
+    def wait_all(self):
+        self.st.add("s_waitcnt lgkmcnt(0)", "wait", wait=0)
+        self.pending.clear()
+
+
+def deal(ops, lo, hi, nslots):
+    """ops dealt evenly over slots lo .. hi (inclusive), in order."""
+    share = [[] for _ in range(nslots)]
+    n = hi - lo + 1
+    for i, op in enumerate(ops):
+        share[lo + i * n // len(ops)].append(op)
+    return share

@@ -23,6 +23,7 @@
 #include "chill_tiles.h"
 #include "chill_bwd_dkdv_regs.h"
 #include "chill_bwd_dq_regs.h"
+#include "chill_bwd_dq_gen.h"
 
 namespace chill {
 
@@ -389,6 +390,23 @@ int launch_dq_shape(const BwdParams& p, hipStream_t stream) {
     return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
 }
 
+// dQ with register-resident Q and dO (16-bit inputs at head dim 128, long sequences on full grids)
+template <typename E, int D, int MASK_ID>
+int launch_dq_regs2(const BwdParams& p, hipStream_t stream) {
+    constexpr TileConfig cfg = dq_regs2_tile_config(D, Elem<E>::kDType);
+    const int n_q_tiles = cdiv(p.T, cfg.rows);
+    const int64_t total64 = (int64_t)p.B * p.H * n_q_tiles;
+    if (total64 > ((int64_t)1 << 30)) return CHILL_ERR_TOO_LARGE;
+    const int total = (int)total64;
+    void (*kern)(BwdParams, int, int, int) = dq_regs2_kernel<E, D, MASK_ID, 4>;
+    const bool hfb = Mask<MASK_ID>::has_full_blocks(64, cfg.streamed, p.T, p.margs);
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, cfg.lds_bytes) !=
+        hipSuccess)
+        return CHILL_ERR_HIP;
+    hipLaunchKernelGGL(kern, dim3(cdiv(total, 8) * 8), dim3(cfg.waves * 64), cfg.lds_bytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
+    return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
+}
+
 // A launch far too small for the chip: 32 rows per workgroup, the streamed axis split over its waves.
 // PASS 1: dQ (workgroups over query blocks), 2: dK/dV (over key blocks).
 template <typename E, int D, int MASK_ID, int PASS>
@@ -423,8 +441,12 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
         bool small = false;
         constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DQ);
         if constexpr (served) small = bwd_takes_small((long long)p.B * p.H, p.T, D, Elem<E>::kDType, CHILL_PASS_DQ);
+        bool regs2 = false;
+        if constexpr (dq_regs2_is_optional(D, Elem<E>::kDType)) regs2 = dq_takes_regs2(MASK_ID, (long long)p.B * p.H, p.T);
         if (small) {
             if constexpr (served) status = launch_bwd_small<E, D, MASK_ID, 1>(p, stream);
+        } else if (regs2) {
+            if constexpr (dq_regs2_is_optional(D, Elem<E>::kDType)) status = launch_dq_regs2<E, D, MASK_ID>(p, stream);
         } else if constexpr (has_short_row) {
             status = dq_takes_short_row((long long)p.B * p.H, p.T) ? launch_dq_shape<E, D, MASK_ID, true>(p, stream)
                                                                    : launch_dq_shape<E, D, MASK_ID, false>(p, stream);

@@ -203,6 +203,22 @@ constexpr int dq_stages(int mask_id, int D, int dtype, int T) {
     return 3 * 2 * dq_streamed(D, dtype) * D * elem_bytes(dtype) <= 144 * 1024 ? 3 : 2;
 }
 
+// 16-bit inputs at head dim 128 have a second dQ kernel (dq_regs2_kernel): 4 waves, one per SIMD, 64 query rows each
+// with Q and dO in registers, 32-key tiles in four stages, runs of predicate-free tiles in a generated loop
+// (gen_dq_loop.py).  It owns its CU; taken like its dK/dV counterpart for long sequences on grids of at least two
+// workgroups per CU, not for the banded masks.  Measured on dQ alone, against dq_kernel on one box: causal B8 H16
+// T8192 2.71 / 2.90 ms, B2 H8 T8192 0.408 / 0.428, prefix-LM B4 H16 T8192 1.45 / 1.55, full mask fp16 B4 H16 T4096
+// 0.76 / 0.82; but causal B16 H16 T4096 1.63 / 1.62, B8 H8 T4096 0.509 / 0.496, B1 H8 T8192 0.227 / 0.232.
+constexpr int kDqRegs2MinSequence = 8192;
+constexpr int kDqRegs2MinWorkgroups = 2 * 256;
+constexpr bool dq_regs2_is_optional(int D, int dtype) { return dtype != CHILL_F32 && D == 128; }
+constexpr bool dq_takes_regs2(int mask_id, long long batch_heads, int T) {
+    return !mask_is_banded(mask_id) && T >= kDqRegs2MinSequence && batch_heads * ((T + 255) / 256) >= kDqRegs2MinWorkgroups;
+}
+constexpr TileConfig dq_regs2_tile_config(int D, int dtype) {
+    return TileConfig{256, 32, 4, 4 * 2 * 32 * D * elem_bytes(dtype)};
+}
+
 // fp32 at head dim 256 (dq_split_kernel): two waves share a 32-query block; two stages of 32-key K and V
 // tiles, then one 4 KiB slot per wave for the two products of a block.
 constexpr bool dq_is_split(int D, int dtype) { return dtype == CHILL_F32 && D == 256; }
@@ -312,6 +328,10 @@ inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_
         case CHILL_PASS_DQ:
             if (T != kLongSequence && bwd_takes_small(batch_heads, T, D, dtype, CHILL_PASS_DQ)) {
                 *out = TileConfig{32, 32, kFwdSmallWaves, bwd_small_lds_bytes(D, dtype, 1)};
+                return CHILL_OK;
+            }
+            if (dq_regs2_is_optional(D, dtype) && (T == kLongSequence ? !mask_is_banded(mask_id) : dq_takes_regs2(mask_id, batch_heads, T))) {
+                *out = dq_regs2_tile_config(D, dtype);
                 return CHILL_OK;
             }
             *out = dq_tile_config(mask_id, D, dtype, (T != kLongSequence && dq_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);

@@ -39,11 +39,10 @@ import os
 import sys
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-from asm_stream import AGPR, Stream, check_clobbers, check_stream, rng, vr  # noqa: E402
+from asm_stream import AGPR, LGKM_MAX, Sched, Stream, areg, check_clobbers, check_stream, deal, rng, vr  # noqa: E402,F401
 
 # fixed scalar register pairs of the four tile pointers (their halves are added to separately)
 PTR_SGPR = {"q": 88, "do": 90, "lse": 92, "del": 94}
-LGKM_MAX = 15   # the counter of outstanding LDS operations has four bits
 ABLATE = set()  # timing experiments only (--ablate): parts of the loop left out; the results are wrong
 TEMP_SGPRS = ("execsave",)
 SPECIAL_CLOBBERS = ["vcc", "scc", "m0"]
@@ -84,11 +83,6 @@ class Config:
         return AGPR + 16 * (self.CB * self.DB + c * self.DB + db)
 
 
-def areg(base, n):
-    b = base - AGPR
-    return f"a[{b}:{b + n - 1}]"
-
-
 class AblatingStream(Stream):
     """Drops the MFMAs of a timing experiment."""
 
@@ -96,49 +90,6 @@ class AblatingStream(Stream):
         if kind == "mfma" and "mfma" in ABLATE:
             return
         super().add(text, kind, *a, **kw)
-
-
-class Sched:
-    """Emits into a Stream, keeps the order of the LDS reads and computes the waits."""
-
-    def __init__(self, st: Stream, carried=()):
-        self.st = st
-        self.seq = 0
-        self.pending = {}
-        for regs in carried:      # reads of the iteration before that may still be in flight, oldest first
-            self.seq += 1
-            for r in regs:
-                self.pending[r] = self.seq
-
-    def read(self, text, addr, regs):
-        self.st.add(text, "lds", [], regs, lds=True)
-        self.seq += 1
-        for r in regs:
-            self.pending[r] = self.seq
-
-    def need(self, regs):
-        seqs = [self.pending[r] for r in regs if r in self.pending]
-        if not seqs:
-            return
-        last = max(seqs)
-        n = min(self.seq - last, LGKM_MAX)
-        self.st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
-        done = self.seq - n
-        for r in [r for r, s in self.pending.items() if s <= done]:
-            del self.pending[r]
-
-    def wait_upto(self, seq):
-        """All reads up to sequence number `seq` have returned."""
-        n = min(self.seq - seq, LGKM_MAX)
-        if any(s <= seq for s in self.pending.values()):
-            self.st.add(f"s_waitcnt lgkmcnt({n})", "wait", wait=n)
-            done = self.seq - n
-            for r in [r for r, s in self.pending.items() if s <= done]:
-                del self.pending[r]
-
-    def wait_all(self):
-        self.st.add("s_waitcnt lgkmcnt(0)", "wait", wait=0)
-        self.pending.clear()
 
 
 def softmax_pairs(c: Config, st: Stream, blk: int, pairs):
@@ -207,15 +158,6 @@ def dma_ops(c: Config, st: Stream, tgt: int):
             A(f"s_addc_u32 {hi}, {hi}, 0", "salu")
         ops.append(advance)
     return ops
-
-
-def deal(ops, lo, hi, nslots):
-    """ops dealt evenly over slots lo .. hi (inclusive), in order."""
-    share = [[] for _ in range(nslots)]
-    n = hi - lo + 1
-    for i, op in enumerate(ops):
-        share[lo + i * n // len(ops)].append(op)
-    return share
 
 
 class Iteration:

@@ -123,7 +123,7 @@ def test_tile_table():
     assert tile_config(window, 64, torch.bfloat16, _lib.PASS_FWD)["streamed"] == 64
     # banded masks, and every mask at head dims <= 64: 4 waves with a two-stage ring, two or more workgroups per CU
     for p, mask, D, waves in ((_lib.PASS_FWD, window, 64, 4), (_lib.PASS_FWD, window, 128, 4), (_lib.PASS_FWD, causal, 64, 4), (_lib.PASS_FWD, causal, 128, 8),
-                              (_lib.PASS_DQ, window, 128, 4), (_lib.PASS_DQ, causal, 64, 4), (_lib.PASS_DQ, causal, 128, 8)):
+                              (_lib.PASS_DQ, window, 128, 4), (_lib.PASS_DQ, causal, 64, 4)):
         c = tile_config(mask, D, torch.bfloat16, p)
         assert c["waves"] == waves, (p, D, c)
         if waves == 4:
@@ -133,7 +133,7 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_FWD)["lds_bytes"] == 4 * 64 * (272 + 320)
     # short sequences and small grids at head dim 128: the 4-wave shape in forward (T <= 1024) and dQ (T <= 4096)
     for p, T, bh, waves in ((_lib.PASS_FWD, 1024, 128, 4), (_lib.PASS_FWD, 1025, 128, 8), (_lib.PASS_DQ, 4096, 128, 4),
-                            (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_FWD, 8192, 8, 8), (_lib.PASS_FWD, 8192, 16, 8),
+                            (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_DQ, 8191, 128, 8), (_lib.PASS_FWD, 8192, 8, 8), (_lib.PASS_FWD, 8192, 16, 8),
                             (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 2048, 8, 4), (_lib.PASS_DKDV, 2048, 16, 8)):
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
@@ -142,6 +142,12 @@ def test_tile_table():
     for D, rows, waves in ((64, 64, 4), (32, 64, 4)):
         c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV)
         assert (c["rows"], c["waves"]) == (rows, waves), (D, c)
+    # dQ at 16-bit head dim 128 from 8192 keys on, full grids, masks that are not banded: Q and dO in registers
+    regs2 = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 4 * 2 * 32 * 256}
+    assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_DQ) == regs2
+    assert tile_config(causal, 128, torch.float16, _lib.PASS_DQ, seq_len=8192, batch_heads=16) == regs2
+    for mask, T, bh in ((causal, 8191, 128), (causal, 8192, 15), (window, 16384, 128)):
+        assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_DQ, seq_len=T, batch_heads=bh)["rows"] != 256, (mask, T, bh)
     # dK/dV at 16-bit head dim 128: K in registers, two 32-key blocks per wave (256 key rows, 4 waves, 32-row tiles in
     # four stages) for long sequences on a grid of two workgroups per CU, except under banded masks; else the paired kernel
     regs = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 256 * 256 + 4 * (2 * 32 * 256 + 2 * 32 * 4)}
@@ -253,7 +259,7 @@ def test_hand_managed_accumulation_registers(elem):
     # dK/dV with register-resident K at head dim 128 (a0..a255 named by the kernel and its generated loop): the
     # compiler touches no accumulation register there, so what it spills is in scratch memory
     rows = tune.hand_managed_registers(elem, 128)
-    assert len(rows) == 5 and all("dkdv_regs_kernel" in name for name, *_ in rows)
+    assert len(rows) == 10 and sum("dkdv_regs_kernel" in name for name, *_ in rows) == 5 and sum("dq_regs2_kernel" in name for name, *_ in rows) == 5
     for name, compiler_max, hand_min, spilled in rows:
         assert compiler_max == -1 and hand_min == 0, (name, compiler_max, hand_min)
 

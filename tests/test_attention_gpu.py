@@ -443,13 +443,19 @@ DKDV_REGS_CASES = [
     ("full-lens-f16", torch.float16, 2, 16, 16, 4130, ("FullChillMask", ()), (4130, 3000)),
     ("prefix-lm", torch.bfloat16, 2, 16, 16, 4096, ("PrefixLMChillMask", (1024,)), None),
     ("prefix-lm-gqa-ragged", torch.float16, 1, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001,)),
+    # sequences from 8192 on: dQ takes its register-resident kernel (chill_bwd_dq_gen.h, gen_dq_loop.py) as well
+    ("long-causal", torch.bfloat16, 1, 16, 16, 8192, ("CausalChillMask", ()), None),
+    ("long-causal-gqa-lens-f16", torch.float16, 2, 16, 8, 8192, ("CausalChillMask", ()), (8192, 5000)),
+    ("long-full-ragged", torch.bfloat16, 1, 32, 16, 8200, ("FullChillMask", ()), None),
+    ("long-prefix-lm-ragged-lens-f16", torch.float16, 1, 32, 32, 8207, ("PrefixLMChillMask", (1024,)), (8100,)),
 ]
 
 
 @pytest.mark.parametrize("case", DKDV_REGS_CASES, ids=lambda c: c[0])
 def test_dkdv_with_resident_keys_and_generated_loop(case):
-    """The dK/dV kernel that keeps K in registers and runs its predicate-free tiles in a generated loop, on shapes the
-    launcher routes to it (asserted from the tile table): heads of a GQA group one after the other, lens, sequence
+    """The dK/dV kernel that keeps K in registers and runs its predicate-free tiles in a generated loop (and, from 8192
+    keys on, the dQ kernel that does the same with Q and dO), on shapes the launcher routes to them (asserted from the
+    tile table): heads of a GQA group one after the other, lens, sequence
     lengths that leave a ragged last tile, the first tiles of a key block under the mask (run by the ordinary code).
     Same bar as the other backward tests (chill_bwd_dkdv.py:347-508 is what it must equal)."""
     _, dtype, B, H, Hkv, T, m, lens = case
@@ -457,6 +463,9 @@ def test_dkdv_with_resident_keys_and_generated_loop(case):
     mask = make_mask(m)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DKDV, seq_len=T, batch_heads=B * Hkv)
     assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
+    # (dQ has such a kernel too, for sequences from 8192 on: the cases of that length below)
+    cfg = tile_config(mask, D, dtype, _lib.PASS_DQ, seq_len=T, batch_heads=B * H)
+    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192), f"dQ served by {cfg}"
     torch.manual_seed(stable_seed(case[0]))
     q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
     lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)

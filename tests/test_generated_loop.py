@@ -145,3 +145,44 @@ def test_backward_loop_check_catches_a_missing_wait():
     broken = st.ins[:waits[3]] + st.ins[waits[3] + 1:]
     with pytest.raises(SystemExit, match="in flight"):
         genb.check_stream(pro.ins + broken + tail, "a wait removed")
+
+
+_spec_q = importlib.util.spec_from_file_location(
+    "gen_dq_loop", os.path.join(ROOT, "chill-attention_amd", "csrc", "gen_dq_loop.py"))
+genq = importlib.util.module_from_spec(_spec_q)
+_spec_q.loader.exec_module(genq)
+
+
+@pytest.mark.parametrize("elem", ["bf16", "f16"])
+def test_dq_loop_generates_and_declares_what_it_writes(elem):
+    """The generated, software-pipelined loop of the dQ kernel with register-resident Q and dO (csrc/gen_dq_loop.py):
+    every path through the statement passes the hazard check, everything it writes is declared, all 256 accumulation
+    registers are on its clobber list (the compiler must park nothing there), and a steady iteration holds what it
+    is meant to."""
+    c = genq.Config(elem)
+    ins = genq.gen_statement(c)  # raises SystemExit if a hazard rule is broken
+    outs, inputs, clob = genq.operand_lists(c)
+    genq.check_clobbers(ins, outs, clob + genq.SPECIAL_CLOBBERS, c.name)
+    assert {f"a{r}" for r in range(256)} <= set(clob)
+    assert c.nvgpr + 32 + 2 + 16 + 4 <= 256   # its own registers, the two -delta blocks, LSE2, addresses, load offsets
+    st = genq.Stream()
+    genq.gen_body(c, st, 1, first=False)
+    text = [i["text"] for i in st.ins]
+    mf = [t for t in text if t.startswith("v_mfma")]
+    assert len(mf) == 48
+    # A_k and B_k take their B operands from the resident Q (a128 ..) and dO (a192 ..), C_(k-1) accumulates into a0 .. a127
+    assert sum(", a[1" in t and t.split()[1].startswith("v[") for t in mf) >= 16
+    acc = [t.split()[1].rstrip(",") for t in mf if t.split()[1].startswith("a[")]
+    assert len(acc) == 16 and len(set(acc)) == 8
+    # LDS: 8 transposed K operands of the tile before (two reads each), 8 V row chunks, 8 K row chunks of the next tile
+    assert sum(t.startswith("ds_read_b64_tr_b16") for t in text) == 16 and sum(t.startswith("ds_read_b128") for t in text) == 16
+    assert sum(t.startswith("v_exp_f32") for t in text) == 32 and sum(t.startswith("v_mul_f32") for t in text) == 32
+    assert sum(t.startswith(c.cvt) for t in text) == 16 and text.count("s_barrier") == 1
+    assert sum(t.startswith("global_load_lds_dwordx4") for t in text) == 4
+    # the barrier stands behind the last MFMA that reads the tile before, and the loads of the tile three ahead behind it
+    order = [n for n, t in enumerate(text) if t == "s_barrier" or t.startswith("global_load_lds") or "a[0:15], v[" in t or
+             t.split()[1].startswith("a[")]
+    bar = text.index("s_barrier")
+    assert all(n < bar for n, t in enumerate(text) if t.startswith("v_mfma") and t.split()[1].startswith("a["))
+    assert all(n > bar for n, t in enumerate(text) if t.startswith("global_load_lds"))
+    assert order
