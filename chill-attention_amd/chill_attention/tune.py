@@ -72,7 +72,8 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
     pair, read from the code-object metadata hipcc writes (``-S``)."""
     rows = []
     with tempfile.TemporaryDirectory() as tmp:
-        for unit in ("chill_fwd_inst.hip", "chill_bwd_inst.hip"):
+        # (at head dim 128 only the backward has such kernels)
+        for unit in ("chill_fwd_inst.hip", "chill_bwd_inst.hip") if dim == 256 else ("chill_bwd_inst.hip",):
             out = os.path.join(tmp, unit + ".s")
             cmd = ["hipcc", *_HIPFLAGS, f"-I{os.path.join(_ROOT, '..', 'include')}",
                    f"-DCHILL_ELEM={elem}_t", f"-DCHILL_ELEM_NAME={elem}", f"-DCHILL_HEAD_DIM={dim}",
@@ -122,7 +123,8 @@ def hand_managed_registers(elem: str = "bf16", dim: int = 256, macros: dict | No
     and nothing is spilled."""
     text = ""
     with tempfile.TemporaryDirectory() as tmp:
-        for unit in ("chill_fwd_inst.hip", "chill_bwd_inst.hip"):
+        # (at head dim 128 only the backward has such kernels)
+        for unit in ("chill_fwd_inst.hip", "chill_bwd_inst.hip") if dim == 256 else ("chill_bwd_inst.hip",):
             out = os.path.join(tmp, unit + ".s")
             cmd = ["hipcc", *_HIPFLAGS, f"-I{os.path.join(_ROOT, '..', 'include')}",
                    f"-DCHILL_ELEM={elem}_t", f"-DCHILL_ELEM_NAME={elem}", f"-DCHILL_HEAD_DIM={dim}",

@@ -147,7 +147,7 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_DQ) == regs2
     assert tile_config(causal, 128, torch.float16, _lib.PASS_DQ, seq_len=8192, batch_heads=16) == regs2
     for mask, T, bh in ((causal, 8191, 128), (causal, 8192, 15), (window, 16384, 128)):
-        assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_DQ, seq_len=T, batch_heads=bh)["rows"] != 256, (mask, T, bh)
+        assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_DQ, seq_len=T, batch_heads=bh)["streamed"] == 64, (mask, T, bh)
     # dK/dV at 16-bit head dim 128: K in registers, two 32-key blocks per wave (256 key rows, 4 waves, 32-row tiles in
     # four stages) for long sequences on a grid of two workgroups per CU, except under banded masks; else the paired kernel
     regs = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 256 * 256 + 4 * (2 * 32 * 256 + 2 * 32 * 4)}
