@@ -32,9 +32,11 @@ def tile_config(mask, head_dim: int, dtype: torch.dtype, pass_id: int, seq_len: 
     if seq_len is None:
         _lib.check("chill_tile_config", lib.chill_tile_config(mask_id, head_dim, _DTYPES[dtype], pass_id, out))
     else:
+        # (with the mask's arguments: the dK/dV row of a chunkwise mask depends on the chunk size)
+        desc = mask.descriptor()
         _lib.check(
-            "chill_tile_config_for_shape",
-            lib.chill_tile_config_for_shape(mask_id, head_dim, _DTYPES[dtype], pass_id, batch_heads, seq_len, out),
+            "chill_tile_config_for_launch",
+            lib.chill_tile_config_for_launch(ctypes.byref(desc), head_dim, _DTYPES[dtype], pass_id, batch_heads, seq_len, out),
         )
     return {"rows": out[0], "streamed": out[1], "waves": out[2], "lds_bytes": out[3]}
 

@@ -203,9 +203,13 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
         delp = p.delta + b * p.delta_b + hq * p.delta_h + q0;
     };
     // Iterations [it, it + n) that the generated loop may run for this wave: the wave's tiles are predicate-free,
-    // and the tiles issued meanwhile (three ahead each) lie in the same query head and exist in full.
+    // and the tiles issued meanwhile (three ahead each) lie in the same query head and exist in full.  In the
+    // last query head of the group the run may go on to the workgroup's last tile when all tiles exist in full:
+    // its last iterations, which would request tiles past the end, take the loop's bodies that request nothing.
     const int run_first = imax(ta, fa);
     const int run_end = imin(imin(tb, fb), imin(n_tiles - (LA + 1), p.T / TQS - wg.start - (LA + 1)));
+    const bool tail_ok = (wg.start + n_tiles) * TQS <= p.T;
+    const int run_end_last = tail_ok ? imin(imin(tb, fb), n_tiles) : run_end;
 
     int st_cur = NS - 1;
     int st_issue = LA;
@@ -213,7 +217,11 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
     for (int it = 0; it < n_iters; it++) {
         if constexpr (kGen) {
             const int t_next = tile + 1 == n_tiles ? 0 : tile + 1;
-            int cnt = (t_next >= run_first) ? run_end - t_next : 0;
+            const bool last_head = it >= n_iters - n_tiles;
+            const int r_end = last_head ? run_end_last : run_end;
+            int cnt = (t_next >= run_first) ? r_end - t_next : 0;
+            // iterations of the run that would request a tile past the workgroup's last
+            const unsigned tailn = uniform((unsigned)imax(0, r_end - (n_tiles - (LA + 1))));
             if (cnt >= 2 && p.scale_log2 != 0.f) {
                 const ET *qp, *dop;
                 const float *lsep, *delp;
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
         a_qrow[0], a_qrow[1], a_qrow[2], a_qrow[3], a_qrow[4], a_qrow[5], a_qrow[6], a_qrow[7], a_qtr[0][0],            \
         a_qtr[0][1], a_qtr[1][0], a_qtr[1][1], a_qtr[2][0], a_qtr[2][1], a_qtr[3][0], a_qtr[3][1], a_vrow[0],           \
         a_vrow[1], a_vrow[2], a_vrow[3], a_vrow[4], a_vrow[5], a_vrow[6], a_vrow[7], a_vec, load_q.goff[0],             \
-        load_q.goff[1], load_do.goff[0], load_do.goff[1], lane4, scale_s, dmabase, vecdma, qstep, dostep, vecwave, st0
+        load_q.goff[1], load_do.goff[0], load_do.goff[1], lane4, scale_s, dmabase, vecdma, qstep, dostep, vecwave, st0, tailn
 #define CHILL_DKDV_LOOP_CALL(loop, ...) loop(__VA_ARGS__)
                 if constexpr (std::is_same<E, bf16_t>::value) {
                     CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_BF16_128, CHILL_DKDV_LOOP_ARGS);

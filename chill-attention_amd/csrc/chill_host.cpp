@@ -121,19 +121,33 @@ int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, i
     return chill_tile_config_for_shape(mask_id, D, dtype, pass, 1, kLongSequence, out);
 }
 
-int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
-                                int32_t T, int32_t out[4]) {
+static int report_tile_config(int mask_id, long long mask_arg0, int32_t D, int32_t dtype, int32_t pass,
+                              int64_t batch_heads, int32_t T, int32_t out[4]) {
     if (out == nullptr) return CHILL_ERR_NULL_POINTER;
     if (!mask_id_served(mask_id)) return CHILL_ERR_BAD_MASK;
     if (T < 1 || batch_heads < 1) return CHILL_ERR_BAD_ARGUMENT;
     TileConfig c;
-    int st = tile_config(mask_id, D, dtype, pass, batch_heads, T, &c);
+    int st = tile_config(mask_id, mask_arg0, D, dtype, pass, batch_heads, T, &c);
     if (st != CHILL_OK) return st;
     out[0] = c.rows;
     out[1] = c.streamed;
     out[2] = c.waves;
     out[3] = c.lds_bytes;
     return CHILL_OK;
+}
+
+int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
+                                int32_t T, int32_t out[4]) {
+    // (a mask id alone: the row of a mask whose arguments do not change the route)
+    return report_tile_config(mask_id, 1, D, dtype, pass, batch_heads, T, out);
+}
+
+int chill_tile_config_for_launch(const ChillMaskDesc* mask, int32_t D, int32_t dtype, int32_t pass,
+                                 int64_t batch_heads, int32_t T, int32_t out[4]) {
+    MaskArgs a;
+    int st = lower_mask(mask, &a);
+    if (st != CHILL_OK) return st;
+    return report_tile_config(mask->id, a.a0, D, dtype, pass, batch_heads, T, out);
 }
 
 const char* chill_status_string(int32_t status) {

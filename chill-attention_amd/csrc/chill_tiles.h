@@ -289,8 +289,15 @@ constexpr int kDkdvRegsBlocks128 = 2;
 constexpr int kDkdvRegsMinSequence = 4096;
 constexpr int kDkdvRegsMinWorkgroups = 2 * 256;
 constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && D == 128 && !CHILL_TUNE_DKDV_R64; }
-constexpr bool dkdv_takes_regs(int mask_id, long long batch_kv_heads, int T) {
-    return !mask_is_banded(mask_id) && T >= kDkdvRegsMinSequence &&
+// Banded masks take it only when a wave's 64 key rows lie in one chunk, so that its tiles are all predicate-free
+// and all alike: chunkwise masks whose chunk size is a multiple of 64 (`mask_arg0` = the mask's first argument;
+// measured at head dim 128, T = 8192 and 16384: chunks of 64 / 128 / 256 / 1024 rows -5 / -8 / -13 / -16 %, chunks
+// of 96 rows +13 %, sliding windows of 64 .. 512 rows +32 .. +60 %, of 1024 rows and more +-1 %).
+constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0) {
+    return mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0;
+}
+constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, long long batch_kv_heads, int T) {
+    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0)) && T >= kDkdvRegsMinSequence &&
            batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >= kDkdvRegsMinWorkgroups;
 }
 
@@ -314,7 +321,9 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype, bool small_
 
 // batch_heads = B * H and T = sequence length of the launch (the forward and dQ rows depend on them);
 // T = kLongSequence for the row of long sequences on a full chip.
-inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_heads, int T, TileConfig* out) {
+// mask_arg0 = the mask's first argument (the dK/dV row of chunkwise masks depends on the chunk size).
+inline int tile_config(int mask_id, long long mask_arg0, int D, int dtype, int pass, long long batch_heads, int T,
+                       TileConfig* out) {
     if (dtype != CHILL_F32 && dtype != CHILL_F16 && dtype != CHILL_BF16) return CHILL_ERR_BAD_DTYPE;
     if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
     switch (pass) {
@@ -344,7 +353,8 @@ inline int tile_config(int mask_id, int D, int dtype, int pass, long long batch_
             }
             // (the row of long sequences on a full chip: the generated loop where there is one)
             *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T),
-                                    T == kLongSequence ? !mask_is_banded(mask_id) : dkdv_takes_regs(mask_id, batch_heads, T));
+                                    T == kLongSequence ? (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0))
+                                                       : dkdv_takes_regs(mask_id, mask_arg0, batch_heads, T));
             return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }

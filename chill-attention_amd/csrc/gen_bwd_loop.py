@@ -184,8 +184,10 @@ class Iteration:
         return out
 
     def generate(self, st: Stream, s: int, with_dma=True, with_prefetch=True, with_barrier=True):
-        """Returns the ring units that hold the Q chunks of the next iteration."""
+        """Returns the ring units that hold the Q chunks of the next iteration.  Without `with_dma` this is an
+        iteration of a run's tail: it requests no tile, and its barrier waits for every tile still on its way."""
         c = self.c
+        self.tail = not with_dma
         nxt, tgt = (s + 1) % c.NSTG, (s + 3) % c.NSTG
         NS = c.slots
         carried = [regs for _, _, regs in self.prefetch_reads(c, s, self.q_units)]
@@ -307,7 +309,19 @@ class Iteration:
         place(pack_ops(c, st, 0, range(0, 4)) + pack_ops(c, st, 1, range(0, 4)), P0_LO, P0_HI)
         place(product_ops(c, st, 0, range(8, 16)) + product_ops(c, st, 1, range(8, 16)), G1_LO, G1_HI)
         place(pack_ops(c, st, 0, range(4, 8)) + pack_ops(c, st, 1, range(4, 8)), P1_LO, P1_HI)
-        scalar = deal(dma_ops(c, st, tgt), 0, 15, NS) if with_dma and "dma" not in ABLATE else [[] for _ in range(NS)]
+        if with_dma and "dma" not in ABLATE:
+            scalar = deal(dma_ops(c, st, tgt), 0, 15, NS)
+        elif "dma" not in ABLATE:
+            # (the vector instructions behind the score MFMAs count on the issue slots the tile loads take)
+            pads = []
+            for op in dma_ops(c, count := Stream(), tgt):
+                before = len(count.ins)
+                op()
+                n_ins = len(count.ins) - before
+                pads.append(lambda n_ins=n_ins: st.add(f"s_nop {n_ins - 1}", "nop", nops=n_ins))
+            scalar = deal(pads, 0, 15, NS)
+        else:
+            scalar = [[] for _ in range(NS)]
 
         next_q = {}
         READS_PER_SLOT = 3
@@ -394,12 +408,13 @@ class Iteration:
         c = self.c
         assert not any(k[0] in ("do", "dot", "qt") for k, _ in queue), "reads of the tile behind the barrier"
         sch.wait_upto(last_tile_read)
+        sfx = f"t{s}" if self.tail else f"{s}"
         st.add("s_cmp_eq_u32 %[cnt], 1", "salu")
-        st.add(f"s_cbranch_scc1 .Lnobar{s}%=", "salu")
-        st.add(f"s_waitcnt vmcnt({c.loads_per_tile})", "wait")
+        st.add(f"s_cbranch_scc1 .Lnobar{sfx}%=", "salu")
+        st.add(f"s_waitcnt vmcnt({0 if self.tail else c.loads_per_tile})", "wait")
         if "barrier" not in ABLATE:
             st.add("s_barrier", "salu")
-        st.add(f".Lnobar{s}%=:", "label", nops=0)
+        st.add(f".Lnobar{sfx}%=:", "label", nops=0)
 
 
 def find_steady_state(c: Config):
@@ -458,7 +473,7 @@ def gen_statement(c: Config):
     for s in range(1, c.NSTG):
         A(f"s_cmp_eq_u32 %[st0], {s}", "salu")
         A(f"s_cbranch_scc1 .Lpro{s}%=", "salu")
-    bodies, pros = [], []
+    bodies, pros, tails = [], [], []
     for s in range(c.NSTG):
         pro = Stream()
         pro.add(f".Lpro{s}%=:", "label", nops=0)
@@ -468,6 +483,9 @@ def gen_statement(c: Config):
         sch = Sched(pro)
         for text, regs in its[s].reads_for_stage(s):
             sch.read(text, None, regs)
+        # a run that starts inside its tail (at most `tailn` iterations, none of which requests a tile)
+        pro.add("s_cmp_le_u32 %[cnt], %[tailn]", "salu")
+        pro.add(f"s_cbranch_scc1 .Ltbody{s}%=", "salu")
         pro.add(f"s_branch .Lbody{s}%=", "salu")
         pros.append(pro)
         body = AblatingStream()
@@ -475,24 +493,42 @@ def gen_statement(c: Config):
         nq = its[s].generate(body, s)
         assert nq == cycle[(s + 1) % n] and its[s].prefetch_order == orders[s % n]
         body.add("s_sub_u32 %[cnt], %[cnt], 1", "salu")
-        body.add("s_cmp_eq_u32 %[cnt], 0", "salu")
-        body.add("s_cbranch_scc1 .Lexit%=", "salu")
+        body.add("s_cmp_le_u32 %[cnt], %[tailn]", "salu")
+        body.add(f"s_cbranch_scc1 .Ltsel{(s + 1) % c.NSTG}%=", "salu")
         if s == c.NSTG - 1:
             body.add("s_branch .Lbody0%=", "salu")
         bodies.append(body)
+        # the same iteration for the last `tailn` tiles of a run that ends with the workgroup's last tile: the
+        # tiles three ahead do not exist
+        tb = AblatingStream()
+        tb.add(f".Ltsel{s}%=:", "label", nops=0)
+        tb.add("s_cmp_eq_u32 %[cnt], 0", "salu")
+        tb.add("s_cbranch_scc1 .Lexit%=", "salu")
+        tb.add(f".Ltbody{s}%=:", "label", nops=0)
+        nq = its[s].generate(tb, s, with_dma=False)
+        assert nq == cycle[(s + 1) % n] and its[s].prefetch_order == orders[s % n]
+        tb.add("s_sub_u32 %[cnt], %[cnt], 1", "salu")
+        if s == c.NSTG - 1:
+            tb.add("s_branch .Ltsel0%=", "salu")
+        tails.append(tb)
     tail = Stream()
     tail.add(".Lexit%=:", "label", nops=0)
     tail.add("s_waitcnt lgkmcnt(0)", "wait", wait=0)
-    # the hazards of every path: a prologue, its body, the next body, the exit
+    # the hazards of every path: a prologue, its body, the next body, the exit; the same through the tail
     for s in range(c.NSTG if not ABLATE else 0):
-        n = (s + 1) % c.NSTG
-        check_stream(pros[s].ins + bodies[s].ins + bodies[n].ins + bodies[(n + 1) % c.NSTG].ins + tail.ins,
-                     f"{c.name} (from stage {s})")
-        check_stream(pros[s].ins + bodies[s].ins + tail.ins, f"{c.name} (one iteration, stage {s})")
+        n1, n2 = (s + 1) % c.NSTG, (s + 2) % c.NSTG
+        for name, path in (("from stage", pros[s].ins + bodies[s].ins + bodies[n1].ins + bodies[n2].ins + tail.ins),
+                           ("one iteration, stage", pros[s].ins + bodies[s].ins + tail.ins),
+                           ("into the tail, stage", pros[s].ins + bodies[s].ins + tails[n1].ins + tails[n2].ins + tail.ins),
+                           ("tail only, stage", pros[s].ins + tails[s].ins + tails[n1].ins + tail.ins),
+                           ("one tail iteration, stage", pros[s].ins + tails[s].ins + tail.ins)):
+            check_stream(path, f"{c.name} ({name} {s})")
     # the first prologue follows the dispatch directly
     out.ins += pros[0].ins
     for s in range(c.NSTG):
         out.ins += bodies[s].ins
+    for s in range(c.NSTG):
+        out.ins += tails[s].ins
     for s in range(1, c.NSTG):
         out.ins += pros[s].ins
     out.ins += tail.ins
@@ -518,7 +554,7 @@ def operand_lists(c: Config):
         ins.append((f"vrow{j}", "v"))
     for n in ("vec", "gq0", "gq1", "gdo0", "gdo1", "lane4"):
         ins.append((n, "v"))
-    for n in ("scale", "dmabase", "vecdma", "qstep", "dostep", "vecwave", "st0"):
+    for n in ("scale", "dmabase", "vecdma", "qstep", "dostep", "vecwave", "st0", "tailn"):
         ins.append((n, "s"))
     # the vector registers of the statement's own, and the accumulation registers of dV^T and dK^T (which
     # the kernel names itself everywhere: the compiler keeps out of them)

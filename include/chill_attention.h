@@ -212,6 +212,14 @@ int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, i
 int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
                                 int32_t T, int32_t out[4]);
 
+/* The same for one launch with its mask: the dK/dV row of a chunkwise mask depends on the chunk size (with
+ * chunks of a multiple of 64 rows a wave's key rows lie in one chunk, no block inside its band is partly
+ * masked, and the launch takes the kernel with the generated loop at head dim 128;
+ * chill_tile_config_for_shape reports the row of the other chunk sizes).
+ * Counterpart of the autotuner's key, which includes the mask's constants (autotune.py:129-240). */
+int chill_tile_config_for_launch(const ChillMaskDesc* mask, int32_t D, int32_t dtype, int32_t pass,
+                                 int64_t batch_heads, int32_t T, int32_t out[4]);
+
 /* Number of unmasked (q, k) pairs with q, k < T, closed form per mask — the numerator of the
  * effective-FLOP metric (benchmark/benchmark.py:271-276 takes it from the dense mask). */
 int64_t chill_mask_nnz(const ChillMaskDesc* mask, int32_t T);

@@ -157,6 +157,23 @@ def test_tile_table():
     for mask, T, bh in ((causal, 4095, 128), (causal, 4096, 31), (window, 8192, 128), (window, None, 1 << 20)):
         c = tile_config(mask, 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
         assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
+    # chunkwise masks whose chunks are a multiple of a wave's 64 key rows (no partly masked block inside the band) take
+    # it too; other chunk sizes do not, nor does the report that is not told the mask's arguments
+    for chunk, T, bh, row in ((128, 16384, 64, regs), (64, 4096, 32, regs), (1024, 8192, 64, regs), (192, 4096, 32, regs)):
+        assert tile_config(ca.ChunkwiseChillMask(chunk, 2), 128, torch.float16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh) == row
+    for mask, T, bh in ((ca.ChunkwiseChillMask(96, 3), 8192, 64), (ca.ChunkwiseChillMask(32, 3), 8192, 64), (ca.ChunkwiseChillMask(128, 2), 4095, 64),
+                        (ca.ChunkwiseChillMask(128, 2), 4096, 31), (ca.ChunkwiseChillMask(128, 2), None, 1 << 20)):
+        c = tile_config(mask, 128, torch.float16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
+        assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
+    out4 = (ctypes.c_int32 * 4)()
+    assert _lib.lib.chill_tile_config_for_shape(3, 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == 0 and out4[0] == 128
+    desc = ca.ChunkwiseChillMask(128, 2).descriptor()
+    assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == 0
+    assert list(out4) == [regs["rows"], regs["streamed"], regs["waves"], regs["lds_bytes"]]
+    assert _lib.lib.chill_tile_config_for_launch(None, 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == -1
+    assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, None) == -1
+    desc.nargs = 1
+    assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == -4
     assert 2 * tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV)["lds_bytes"] <= 160 * 1024
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
     assert tq == 32 * waves and tk % 32 == 0

@@ -448,6 +448,12 @@ DKDV_REGS_CASES = [
     ("long-causal-gqa-lens-f16", torch.float16, 2, 16, 8, 8192, ("CausalChillMask", ()), (8192, 5000)),
     ("long-full-ragged", torch.bfloat16, 1, 32, 16, 8200, ("FullChillMask", ()), None),
     ("long-prefix-lm-ragged-lens-f16", torch.float16, 1, 32, 32, 8207, ("PrefixLMChillMask", (1024,)), (8100,)),
+    # chunks of a multiple of a wave's 64 key rows: every block inside the band is predicate-free (dQ keeps its ordinary kernel);
+    # runs that start in the middle of a workgroup's tiles and end before its last, a GQA group, a ragged end
+    ("chunkwise-128x2-f16", torch.float16, 1, 16, 16, 8192, ("ChunkwiseChillMask", (128, 2)), None),
+    ("chunkwise-64x4-gqa-lens", torch.bfloat16, 4, 16, 8, 4096, ("ChunkwiseChillMask", (64, 4)), (4096, 3000, 77, 4001)),
+    ("chunkwise-1024x1-ragged-f16", torch.float16, 1, 32, 32, 4140, ("ChunkwiseChillMask", (1024, 1)), None),
+    ("chunkwise-192x0", torch.bfloat16, 1, 32, 32, 4096, ("ChunkwiseChillMask", (192, 0)), None),
 ]
 
 
@@ -465,7 +471,8 @@ def test_dkdv_with_resident_keys_and_generated_loop(case):
     assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
     # (dQ has such a kernel too, for sequences from 8192 on: the cases of that length below)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DQ, seq_len=T, batch_heads=B * H)
-    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192), f"dQ served by {cfg}"
+    banded = m[0] == "ChunkwiseChillMask"
+    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192 and not banded), f"dQ served by {cfg}"
     torch.manual_seed(stable_seed(case[0]))
     q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
     lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)

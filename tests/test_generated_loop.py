@@ -129,6 +129,31 @@ def test_backward_loop_generates_and_declares_what_it_writes(elem):
     assert len(nxt) == 4 + 8 + 8
 
 
+def test_backward_loop_tail_requests_no_tile():
+    """The iterations a run ends with when it reaches the workgroup's last tile (the tiles three ahead do not exist):
+    the same 64 MFMAs, LDS reads and vector work, no tile load and no pointer moved on, and the barrier waits for
+    every tile still on its way.  The statement holds one such body per stage and enters them by the count."""
+    c = genb.Config("bf16")
+    cycle, orders = genb.find_steady_state(c)
+    it = genb.SteadyIteration(c, cycle[0], orders[-1])
+    body, tail = genb.Stream(), genb.Stream()
+    assert it.generate(body, 0) == it.generate(tail, 0, with_dma=False)
+    kinds = lambda st, k: [i["text"] for i in st.ins if i["kind"] == k]  # noqa: E731
+    assert kinds(body, "mfma") == kinds(tail, "mfma") and kinds(body, "valu") == kinds(tail, "valu")
+    assert [t for t in kinds(body, "lds")] == [t for t in kinds(tail, "lds")]
+    text = [i["text"] for i in tail.ins]
+    assert not any("global_load" in t or "s_add_u32" in t or "s_addc_u32" in t for t in text)
+    assert "s_waitcnt vmcnt(0)" in text and f"s_waitcnt vmcnt({c.loads_per_tile})" not in text
+    assert f"s_waitcnt vmcnt({c.loads_per_tile})" in [i["text"] for i in body.ins]
+    # (the padding keeps the distance between the score MFMAs and the vector work that reads them)
+    assert sum(i["nops"] for i in tail.ins) >= sum(i["nops"] for i in body.ins) - 4
+    whole = [i["text"] for i in genb.gen_statement(c)]
+    for s in range(c.NSTG):
+        assert f".Ltbody{s}%=:" in whole and f".Ltsel{s}%=:" in whole
+    assert whole.count("s_cmp_le_u32 %[cnt], %[tailn]") == 2 * c.NSTG
+    assert ("tailn", "s") in genb.operand_lists(c)[1]
+
+
 def test_backward_loop_check_catches_a_missing_wait():
     """The same stream with one of its computed waits removed does not pass."""
     c = genb.Config("bf16")
