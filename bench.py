@@ -38,10 +38,10 @@ PEAK_HBM_GBS = 8000.0
 # sources it was measured on (kernel_sources_digest below); with other sources the line reports null.
 TRAFFIC_SOURCE = "profiles/c3_causal_bf16_fwd_bwd_kernels.md"
 MEASURED_TRAFFIC = {
-    ("C3", "chill_fwd"): (599825 * 2.0 + 352257) * 1024,
-    ("C3", "chill_bwd_delta"): (262171 * 2.0 + 4202) * 1024,
-    ("C3", "chill_bwd_dkdv"): (528630 * 2.0 + 524288) * 1024,
-    ("C3", "chill_bwd_dq"): (752864 * 2.0 + 262144) * 1024,
+    ("C3", "chill_fwd"): (599150 * 2.0 + 344064) * 1024,
+    ("C3", "chill_bwd_delta"): (262171 * 2.0 + 4198) * 1024,
+    ("C3", "chill_bwd_dkdv"): (823780 * 2.0 + 577536) * 1024,
+    ("C3", "chill_bwd_dq"): (739996 * 2.0 + 277979) * 1024,
 }
 
 
