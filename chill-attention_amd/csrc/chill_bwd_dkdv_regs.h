@@ -14,12 +14,12 @@
 // CB = 1, D = 256 (512-byte rows) is the shipped dK/dV kernel of that shape: 2 x 8 accumulator blocks
 // are exactly the 256 accumulation registers, which the compiler cannot keep there by itself (its
 // version of this kernel spills 2400 registers to scratch and runs 40x slower).
-// CB = 2, D = 64 / 128 is a sweep candidate (-DCHILL_TUNE_DKDV_R64=1): every streamed operand fetched
-// from LDS feeds two MFMAs and K is never re-read, 0.75 KiB of LDS traffic per MFMA where the paired
-// kernel needs 1.5 KiB.  On the causal bf16 B8 H16 T8192 D128 workload it is as fast as the paired
-// kernel (4.2-4.6 ms, box to box), not faster: with one wave per SIMD the vector work hides only
-// behind the wave's own MFMAs (0.9 ms of it stays exposed) and the per-tile synchronisation costs
-// as much again, so the table keeps the paired kernel there.
+// CB = 2, D = 128 is the dK/dV kernel of long sequences at that head dim (chill_tiles.h: dkdv_takes_regs):
+// every streamed operand fetched from LDS feeds two MFMAs and K is never re-read, 76 LDS reads per 64
+// MFMAs where the paired kernel needs 146.  Its runs of predicate-free tiles go through a generated,
+// hazard-checked loop (gen_bwd_loop.py -> chill_bwd_loop.inc); with the compiler's schedule the shape was
+// no faster than the paired kernel (a lone wave hides its vector work only behind its own MFMAs).  The
+// same shape at D = 64 remains a sweep candidate (-DCHILL_TUNE_DKDV_R64=1, compiler-scheduled).
 //
 // Every translation unit that instantiates this kernel is checked (tests/test_abi.py) for the
 // compiler keeping out of the accumulation registers the kernel names itself.

@@ -280,11 +280,11 @@ constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
 // 16-bit inputs at head dim 128 have both kernels: the paired one, and dkdv_regs_kernel with two blocks per wave,
 // whose runs of predicate-free tiles go through a generated loop (gen_bwd_loop.py).  The latter owns its CU (130 KiB of
 // LDS, 512 registers per wave) and pays more before and after its loop (K into registers, V negated in LDS, no second
-// workgroup to hide behind): it is taken for long sequences on a grid of at least two workgroups per CU, and not
-// for the banded masks, whose runs are a few tiles long.  Measured on dK/dV alone, against the paired kernel:
+// workgroup to hide behind): it is taken for long sequences on a grid of at least two workgroups per CU, and of
+// the banded masks only for those named below.  Measured on dK/dV alone, against the paired kernel:
 // causal B8 H16 T8192 3.63 / 4.06 ms, B16 H16 T4096 2.18 / 2.27, B2 H8 T8192 0.547 / 0.591, full mask fp16 B4 H16
 // T4096 0.98 / 1.16, prefix-LM B4 H16 T8192 1.91 / 2.16; but causal B1 H8 T8192 0.368 / 0.318, B4 H16 T2048
-// 0.227 / 0.197, sliding window 512 at T8192 0.65 / 0.49; chunkwise (128, 2) fp16 B2 H32 T16384 0.74 / 0.75.
+// 0.227 / 0.197, sliding window 512 at T8192 0.65 / 0.49.
 constexpr int kDkdvRegsBlocks128 = 2;
 constexpr int kDkdvRegsMinSequence = 4096;
 constexpr int kDkdvRegsMinWorkgroups = 2 * 256;

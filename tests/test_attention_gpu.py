@@ -533,6 +533,28 @@ def test_gradients_through_strided_and_fp32_dout():
         torch.testing.assert_close(got, want.half(), atol=5e-3, rtol=1e-3)
 
 
+def test_register_resident_backward_on_strided_views():
+    """The long-sequence backward kernels at head dim 128 (K, or Q and dO, in registers; tile pointers that the generated
+    loops move on by a row stride) on [B, T, H, D] storage viewed as [B, H, T, D], a GQA group, and an upstream gradient
+    with a padded row pitch: bit for bit what the same launch gives on contiguous copies."""
+    mask = ca.CausalChillMask()
+    B, H, Hkv, T, D = 2, 16, 8, 8192, 128
+    dtype = torch.bfloat16
+    for pss, cfg_heads in ((_lib.PASS_DKDV, B * Hkv), (_lib.PASS_DQ, B * H)):
+        cfg = tile_config(mask, D, dtype, pss, seq_len=T, batch_heads=cfg_heads)
+        assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
+    torch.manual_seed(11)
+    q = torch.randn(B, T, H, D, device=DEV, dtype=dtype).transpose(1, 2).requires_grad_()
+    k, v = (torch.randn(B, T, Hkv, D, device=DEV, dtype=dtype).transpose(1, 2).requires_grad_() for _ in range(2))
+    dout = torch.randn(B, H, T, 2 * D, device=DEV, dtype=dtype)[..., D:]
+    assert not q.is_contiguous() and not dout.is_contiguous()
+    ca.chill_attention(q, k, v, mask=mask).backward(dout)
+    qc, kc, vc = (x.detach().contiguous().requires_grad_() for x in (q, k, v))
+    ca.chill_attention(qc, kc, vc, mask=mask).backward(dout.contiguous())
+    for name, got, want in (("dq", q.grad, qc.grad), ("dk", k.grad, kc.grad), ("dv", v.grad, vc.grad)):
+        assert torch.equal(got, want), name
+
+
 def test_mask_args_are_runtime_values():
     """Instances of one mask class share one registered op; their arguments reach the kernel at run time."""
     q, k, v = (torch.randn(1, 2, 256, 64, device=DEV, dtype=torch.float16) for _ in range(3))
