@@ -431,6 +431,12 @@ def main():
             kernels[i][0]: max(per_entry[kernels[i][0]] * B * H * D * nnz / (peak * 1e12),
                                alg_bytes[kernels[i][0]] / (PEAK_HBM_GBS * 1e9)) / (k_ms[i] * 1e-3)
             for i in range(len(kernels))},
+        # the matrix work each kernel EXECUTES (dQ recomputes S and dP: 6*D per entry for its algorithmic 2*D)
+        # over its time, as a fraction of the peak
+        "kernel_executed_frac_of_peak": {
+            kernels[i][0]: {"chill_fwd": 4.0, "chill_bwd_dkdv": 8.0, "chill_bwd_dq": 6.0}[kernels[i][0]] * B * H * D * nnz
+            / (k_ms[i] * 1e-3) / (peak * 1e12)
+            for i in range(len(kernels)) if kernels[i][0] != "chill_bwd_delta"},
         "sustained": sustained,
         "sm_clock_mhz": sustained["sm_clock_mhz"] if sustained else None,
         "operator_ms_per_step": op_ms,
