@@ -4,8 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3] [--mode fwd+bwd|fwd]
 
 One "step" is one pass of the hot path over one batch of synthetic input that is already
-resident in HBM: forward (chill_fwd) and, in fwd+bwd mode, the backward launches (chill_bwd_delta,
-chill_bwd_dkdv, chill_bwd_dq), all through the C ABI on pre-allocated buffers.  Prints ONE JSON line.
+resident in HBM: forward (chill_fwd) and, in fwd+bwd mode, the backward launches (chill_bwd_dq_delta, which
+computes delta on its way, then chill_bwd_dkdv: what the operator's backward launches), all through the C ABI
+on pre-allocated buffers.  Prints ONE JSON line.
 
   value      effective TFLOP/s over unmasked score entries (4*B*H*D*nnz forward, 2.5x for backward)
   roofline   for the kernel that takes the largest share of the step: algorithmic FLOPs per launch
@@ -207,10 +208,22 @@ class Runner:
             ctypes.c_void_p(self.lse.data_ptr()), self.s_lse, ctypes.c_void_p(self.delta.data_ptr()), self.s_delta,
             None, 0, B, H, Hkv, T, D, self.dtype, self.sm_scale, ctypes.byref(self.desc), ctypes.c_void_p(self.stream)))
 
-    def kernels(self, mode):
+    def dq_delta_(self):
+        B, H, Hkv, T, D = self.shape
+        L = self._lib
+        L.check("chill_bwd_dq_delta", L.lib.chill_bwd_dq_delta(
+            self._r("q"), self._r("k"), self._r("v"), self._r("o"), self._r("do"), self._r("dq"),
+            ctypes.c_void_p(self.lse.data_ptr()), self.s_lse, ctypes.c_void_p(self.delta.data_ptr()), self.s_delta,
+            None, 0, B, H, Hkv, T, D, self.dtype, self.sm_scale, ctypes.byref(self.desc), ctypes.c_void_p(self.stream)))
+
+    def kernels(self, mode, separate_delta=False):
+        """The launches of one step.  separate_delta: the backward as the three launches of the reference's
+        structure (delta, dK/dV, dQ) instead of the two the operator uses."""
         ks = [("chill_fwd", self.fwd)]
-        if mode == "fwd+bwd":
+        if mode == "fwd+bwd" and separate_delta:
             ks += [("chill_bwd_delta", self.delta_), ("chill_bwd_dkdv", self.dkdv), ("chill_bwd_dq", self.dq_)]
+        elif mode == "fwd+bwd":
+            ks += [("chill_bwd_dq_delta", self.dq_delta_), ("chill_bwd_dkdv", self.dkdv)]
         return ks
 
 
@@ -263,6 +276,8 @@ def main():
     ap.add_argument("--workload", default="C3", choices=sorted(WORKLOADS))
     ap.add_argument("--mode", default="fwd+bwd", choices=["fwd", "fwd+bwd"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--separate-delta", action="store_true",
+                    help="time the backward as three launches (delta, dK/dV, dQ) instead of the operator's two")
     ap.add_argument("--sustained-seconds", type=float, default=3.0,
                     help="length of the continuous loop behind the `sustained` figure (0: leave it out)")
     ap.add_argument("--sigma", type=float, default=None,
@@ -297,7 +312,7 @@ def main():
     torch.cuda.set_device(dev)
     q, k, v, do = make_inputs(torch, B, H, T, D, dtype, seed, sigma, dev)
     run = Runner(torch, ca, mask, q, k, v, do, D ** -0.5)
-    kernels = run.kernels(mode)
+    kernels = run.kernels(mode, args.separate_delta)
 
     if args.copy_probe:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
@@ -376,7 +391,7 @@ def main():
     # algorithmic FLOPs per launch: forward 4*D per unmasked entry (2 GEMMs); of the backward's
     # 10*D (5 GEMMs: S, dP, dV, dK, dQ) the dK/dV kernel is charged S, dP, dV, dK = 8*D and the dQ
     # kernel dQ = 2*D (its own S and dP are recomputation, not algorithmic work)
-    per_entry = {"chill_fwd": 4.0, "chill_bwd_dkdv": 8.0, "chill_bwd_dq": 2.0, "chill_bwd_delta": 0.0}
+    per_entry = {"chill_fwd": 4.0, "chill_bwd_dkdv": 8.0, "chill_bwd_dq": 2.0, "chill_bwd_dq_delta": 2.0, "chill_bwd_delta": 0.0}
     es = 4 if dname == "f32" else 2
     dom = max(range(len(kernels)), key=lambda i: k_ms[i])
     dom_name = kernels[dom][0]
@@ -385,6 +400,7 @@ def main():
         "chill_bwd_delta": 2.0 * B * H * T * D * es + 4.0 * B * H * T,
         "chill_bwd_dkdv": 6.0 * B * H * T * D * es + 8.0 * B * H * T,
         "chill_bwd_dq": 5.0 * B * H * T * D * es + 8.0 * B * H * T,
+        "chill_bwd_dq_delta": 6.0 * B * H * T * D * es + 8.0 * B * H * T,
     }
     alg_flops = per_entry[dom_name] * B * H * D * nnz
     # the roof that bounds the kernel: max(FLOPs / peak, algorithmic bytes / HBM bandwidth)
@@ -434,7 +450,7 @@ def main():
         # the matrix work each kernel EXECUTES (dQ recomputes S and dP: 6*D per entry for its algorithmic 2*D)
         # over its time, as a fraction of the peak
         "kernel_executed_frac_of_peak": {
-            kernels[i][0]: {"chill_fwd": 4.0, "chill_bwd_dkdv": 8.0, "chill_bwd_dq": 6.0}[kernels[i][0]] * B * H * D * nnz
+            kernels[i][0]: {"chill_fwd": 4.0, "chill_bwd_dkdv": 8.0, "chill_bwd_dq": 6.0, "chill_bwd_dq_delta": 6.0}[kernels[i][0]] * B * H * D * nnz
             / (k_ms[i] * 1e-3) / (peak * 1e12)
             for i in range(len(kernels)) if kernels[i][0] != "chill_bwd_delta"},
         "sustained": sustained,

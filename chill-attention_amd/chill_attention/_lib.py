@@ -59,6 +59,8 @@ def load_library(path: str) -> ctypes.CDLL:
         "chill_bwd_delta": (c_int32, [T4, T4, c_void_p, I64_3, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p]),
         "chill_bwd_dq": (c_int32, [T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, I64_3, c_void_p, c_int64,
                                    c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
+        "chill_bwd_dq_delta": (c_int32, [T4, T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, I64_3, c_void_p, c_int64,
+                                         c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
         "chill_bwd_dkdv": (c_int32, [T4, T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, I64_3, c_void_p, c_int64,
                                      c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_float, MD, c_void_p]),
         "chill_bwd_noalloc": (c_int32, [T4, T4, T4, T4, T4, T4, T4, T4, c_void_p, I64_3, c_void_p, c_int64,
@@ -90,7 +92,7 @@ def load_library(path: str) -> ctypes.CDLL:
 
 lib = load_library(LIB_PATH)
 EXPORTED_SYMBOLS = (
-    "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dkdv", "chill_bwd_noalloc", "chill_mask_eval_device",
+    "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dq_delta", "chill_bwd_dkdv", "chill_bwd_noalloc", "chill_mask_eval_device",
     "chill_tile_ranges_device", "chill_mask_eval", "chill_mask_limits", "chill_tile_ranges",
     "chill_mask_is_full_block", "chill_mask_has_full_blocks", "chill_tile_config", "chill_tile_config_for_shape",
     "chill_tile_config_for_launch",
@@ -115,11 +117,11 @@ class EntryPoints(ctypes.Structure):
     of the table, in the order csrc/chill_torch.cpp declares."""
 
     _fields_ = [("magic", ctypes.c_uint64), ("abi_version", ctypes.c_uint32), ("bytes", ctypes.c_uint32)] + [
-        (n, c_void_p) for n in ("fwd", "delta", "dkdv", "dq", "status_string")]
+        (n, c_void_p) for n in ("fwd", "dq_delta", "dkdv", "status_string")]
 
 
 def entry_points(cdll: ctypes.CDLL) -> EntryPoints:
-    names = ("chill_fwd", "chill_bwd_delta", "chill_bwd_dkdv", "chill_bwd_dq", "chill_status_string")
+    names = ("chill_fwd", "chill_bwd_dq_delta", "chill_bwd_dkdv", "chill_status_string")
     return EntryPoints(ENTRY_POINTS_MAGIC, cdll.chill_abi_version(), ctypes.sizeof(EntryPoints),
                        *(ctypes.cast(getattr(cdll, n), c_void_p).value for n in names))
 

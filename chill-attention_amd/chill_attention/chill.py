@@ -181,11 +181,16 @@ def register_chill_mask(mask: ChillMask):
         stream = ctypes.c_void_p(_stream_ptr(q))
         lse_p, delta_p = ctypes.c_void_p(lse.data_ptr()), ctypes.c_void_p(delta.data_ptr())
         with torch.cuda.device(q.device):
+            # dQ first: it computes delta = rowsum(O * dO) of its rows on the way (the reference's separate
+            # preprocessing launch, chill.py:278-290) and leaves it in `delta` for dK/dV
             _lib.check(
-                "chill_bwd_delta",
-                mask_lib.chill_bwd_delta(
-                    ctypes.byref(to), ctypes.byref(tdo), delta_p, _lib.strides3(delta),
-                    batch, heads, T, head_dim, dtype, stream,
+                "chill_bwd_dq_delta",
+                mask_lib.chill_bwd_dq_delta(
+                    ctypes.byref(tq), ctypes.byref(tk), ctypes.byref(tv), ctypes.byref(to), ctypes.byref(tdo),
+                    ctypes.byref(tdq),
+                    lse_p, _lib.strides3(lse), delta_p, _lib.strides3(delta), lens_ptr, lens_stride,
+                    batch, heads, num_kv_heads, T, head_dim, dtype, float(sm_scale),
+                    ctypes.byref(desc), stream,
                 ),
             )
             _lib.check(
@@ -193,15 +198,6 @@ def register_chill_mask(mask: ChillMask):
                 mask_lib.chill_bwd_dkdv(
                     ctypes.byref(tq), ctypes.byref(tk), ctypes.byref(tv), ctypes.byref(tdo),
                     ctypes.byref(tdk), ctypes.byref(tdv),
-                    lse_p, _lib.strides3(lse), delta_p, _lib.strides3(delta), lens_ptr, lens_stride,
-                    batch, heads, num_kv_heads, T, head_dim, dtype, float(sm_scale),
-                    ctypes.byref(desc), stream,
-                ),
-            )
-            _lib.check(
-                "chill_bwd_dq",
-                mask_lib.chill_bwd_dq(
-                    ctypes.byref(tq), ctypes.byref(tk), ctypes.byref(tv), ctypes.byref(tdo), ctypes.byref(tdq),
                     lse_p, _lib.strides3(lse), delta_p, _lib.strides3(delta), lens_ptr, lens_stride,
                     batch, heads, num_kv_heads, T, head_dim, dtype, float(sm_scale),
                     ctypes.byref(desc), stream,

@@ -207,6 +207,24 @@ int chill_bwd_dq(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor
     return kDq[dtype][dim_index(D)](p, mask->id, static_cast<hipStream_t>(stream));
 }
 
+int chill_bwd_dq_delta(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+                       const ChillTensor4* o, const ChillTensor4* d_o, const ChillTensor4* dq,
+                       const float* lse, const int64_t lse_stride[3], float* delta,
+                       const int64_t delta_stride[3], const int32_t* lens, int64_t lens_stride,
+                       int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D, int32_t dtype,
+                       float sm_scale, const ChillMaskDesc* mask, void* stream) {
+    int es = 0;
+    BwdParams p = {};
+    CHILL_TRY(lower_bwd(&p, q, k, v, d_o, lse, lse_stride, delta, delta_stride, lens, lens_stride,
+                        B, H, H_kv, T, D, dtype, sm_scale, mask, &es));
+    CHILL_TRY(lower_tensor(dq, es, &p.sdq));
+    CHILL_TRY(lower_tensor(o, es, &p.so));
+    p.dq = dq->ptr;
+    p.o = o->ptr;
+    p.delta_out = delta;
+    return kDq[dtype][dim_index(D)](p, mask->id, static_cast<hipStream_t>(stream));
+}
+
 int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
                    const ChillTensor4* d_o, const ChillTensor4* dk, const ChillTensor4* dv,
                    const float* lse, const int64_t lse_stride[3], const float* delta,
@@ -225,8 +243,8 @@ int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTens
 }
 
 // ---------------------------------------------------------------------------------------------
-// The whole backward without a workspace from the caller.  The fp32 delta rows, which chill_bwd_delta
-// writes and the two gradient kernels read, live in a device array of this library: each GPU the
+// The whole backward without a workspace from the caller.  The fp32 delta rows, which chill_bwd_dq_delta
+// writes and chill_bwd_dkdv reads, live in a device array of this library: each GPU the
 // library runs on holds its own copy of `scratch` until the process ends.  In host code the array's
 // name is a stand-in, not a device address: the address comes from hipGetSymbolAddress, once per
 // device with that device current, and only that pointer is handed to kernels.
@@ -266,12 +284,11 @@ int chill_bwd_noalloc(const ChillTensor4* q, const ChillTensor4* k, const ChillT
     float* delta = nullptr;
     CHILL_TRY(scratch_of_current_device(&delta));
     const int64_t delta_stride[3] = {(int64_t)H * T, (int64_t)T, 1};
-    // every row of delta is written by the first launch before the other two read it: nothing to clear
-    CHILL_TRY(chill_bwd_delta(o, d_o, delta, delta_stride, B, H, T, D, dtype, stream));
-    CHILL_TRY(chill_bwd_dkdv(q, k, v, d_o, dk, dv, lse, lse_stride, delta, delta_stride, lens, lens_stride, B, H,
-                             H_kv, T, D, dtype, sm_scale, mask, stream));
-    return chill_bwd_dq(q, k, v, d_o, dq, lse, lse_stride, delta, delta_stride, lens, lens_stride, B, H, H_kv, T, D,
-                        dtype, sm_scale, mask, stream);
+    // every row of delta is written by the first launch before the second reads it: nothing to clear
+    CHILL_TRY(chill_bwd_dq_delta(q, k, v, o, d_o, dq, lse, lse_stride, delta, delta_stride, lens, lens_stride, B, H,
+                                 H_kv, T, D, dtype, sm_scale, mask, stream));
+    return chill_bwd_dkdv(q, k, v, d_o, dk, dv, lse, lse_stride, delta, delta_stride, lens, lens_stride, B, H, H_kv, T,
+                          D, dtype, sm_scale, mask, stream);
 }
 
 }  // extern "C"

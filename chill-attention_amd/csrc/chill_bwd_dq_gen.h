@@ -99,6 +99,10 @@ __global__ __launch_bounds__(256) void dq_regs2_kernel(BwdParams p, int n_q_tile
     ET* dqbase = reinterpret_cast<ET*>(p.dq) + b * p.sdq.b + hd * p.sdq.h;
     if (qb >= seq_len) {
         zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(TQ, p.T - qb), tid);
+        if (p.delta_out != nullptr) {
+            // (the dK/dV launch that follows reads delta of every row of the tiles it visits)
+            for (int i = tid; i < imin(TQ, p.T - qb); i += NT) p.delta_out[b * p.delta_b + hd * p.delta_h + qb + i] = 0.f;
+        }
         return;
     }
 
@@ -142,8 +146,12 @@ __global__ __launch_bounds__(256) void dq_regs2_kernel(BwdParams p, int n_q_tile
         load_resident<E, D>(dof, doptr + (int64_t)q0 * p.sdo.t, p.sdo.t, p.T - q0, lane);
         lse_q[c] = 0.f;
         delta_q[c] = 0.f;
-        if (q0 + n < p.T) {
-            lse_q[c] = p.lse[b * p.lse_b + hd * p.lse_h + q0 + n];
+        if (q0 + n < p.T) lse_q[c] = p.lse[b * p.lse_b + hd * p.lse_h + q0 + n];
+        if (p.delta_out != nullptr) {
+            const ET* optr = reinterpret_cast<const ET*>(p.o) + b * p.so.b + hd * p.so.h;
+            delta_q[c] = resident_row_delta<E, D>(dof, optr + (int64_t)q0 * p.so.t, p.so.t, p.T - q0, lane);
+            if (h == 0 && q0 + n < p.T) p.delta_out[b * p.delta_b + hd * p.delta_h + q0 + n] = delta_q[c];
+        } else if (q0 + n < p.T) {
             delta_q[c] = p.delta[b * p.delta_b + hd * p.delta_h + q0 + n];
         }
         // a row that attends to nothing has LSE2 = -inf and only masked entries (score -inf): P = exp2(-inf - 0)

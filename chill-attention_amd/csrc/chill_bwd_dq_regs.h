@@ -59,6 +59,10 @@ __global__ __launch_bounds__(256) void dq_regs_kernel(BwdParams p, int n_q_tiles
     ET* dqbase = reinterpret_cast<ET*>(p.dq) + b * p.sdq.b + hd * p.sdq.h;
     if (qb >= seq_len) {
         zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(TQ, p.T - qb), tid);
+        if (p.delta_out != nullptr) {
+            // (the dK/dV launch that follows reads delta of every row of the tiles it visits)
+            for (int i = tid; i < imin(TQ, p.T - qb); i += NT) p.delta_out[b * p.delta_b + hd * p.delta_h + qb + i] = 0.f;
+        }
         return;
     }
 
@@ -90,8 +94,12 @@ __global__ __launch_bounds__(256) void dq_regs_kernel(BwdParams p, int n_q_tiles
     load_resident<E, D>(qf, qptr + (int64_t)qw * p.sq.t, p.sq.t, p.T - qw, lane);
     load_resident<E, D>(dof, doptr + (int64_t)qw * p.sdo.t, p.sdo.t, p.T - qw, lane);
     float lse_q = 0.f, delta_q = 0.f;
-    if (q_pos < p.T) {
-        lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
+    if (q_pos < p.T) lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
+    if (p.delta_out != nullptr) {
+        const ET* optr = reinterpret_cast<const ET*>(p.o) + b * p.so.b + hd * p.so.h;
+        delta_q = resident_row_delta<E, D>(dof, optr + (int64_t)qw * p.so.t, p.so.t, p.T - qw, lane);
+        if (h == 0 && q_pos < p.T) p.delta_out[b * p.delta_b + hd * p.delta_h + q_pos] = delta_q;
+    } else if (q_pos < p.T) {
         delta_q = p.delta[b * p.delta_b + hd * p.delta_h + q_pos];
     }
     // a row that attends to nothing has LSE2 = -inf and only masked entries (score -inf): P = exp2(-inf - 0)

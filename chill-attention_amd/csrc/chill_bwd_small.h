@@ -85,6 +85,10 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void dq_small_kernel(BwdParams
     if (qb >= seq_len) {
         // rows at or beyond lens[b] receive 0 (the reference relies on the adapter's zero-fill, chill.py:292)
         zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(32, p.T - qb), tid);
+        if (p.delta_out != nullptr) {
+            // (the dK/dV launch that follows reads delta of every row of the tiles it visits)
+            for (int i = tid; i < imin(32, p.T - qb); i += NT) p.delta_out[b * p.delta_b + hd * p.delta_h + qb + i] = 0.f;
+        }
         return;
     }
 
@@ -114,8 +118,13 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void dq_small_kernel(BwdParams
     load_resident<E, D>(dof, doptr + (int64_t)qb * p.sdo.t, p.sdo.t, p.T - qb, lane);
     const int q_pos = qb + n;
     float lse_q = 0.f, delta_q = 0.f;
-    if (q_pos < p.T) {
-        lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
+    if (q_pos < p.T) lse_q = p.lse[b * p.lse_b + hd * p.lse_h + q_pos];
+    if (p.delta_out != nullptr) {
+        // (every wave of the workgroup holds the same 32 rows; the first one writes)
+        const ET* optr = reinterpret_cast<const ET*>(p.o) + b * p.so.b + hd * p.so.h;
+        delta_q = resident_row_delta<E, D>(dof, optr + (int64_t)qb * p.so.t, p.so.t, p.T - qb, lane);
+        if (wave == 0 && (lane >> 5) == 0 && q_pos < p.T) p.delta_out[b * p.delta_b + hd * p.delta_h + q_pos] = delta_q;
+    } else if (q_pos < p.T) {
         delta_q = p.delta[b * p.delta_b + hd * p.delta_h + q_pos];
     }
     OperandOffsets<E, D> ofs;

@@ -737,6 +737,29 @@ __device__ __forceinline__ void load_resident(Resident<E, D>& regs,
     }
 }
 
+// delta of the lane's row, sum over the head dim of O * dO (utils.py:94-217), for a dQ kernel that keeps
+// the row's dO chunks as a resident operand: the same chunks of O are read here, every lane sums its
+// half of the row and the row's two lanes add up.  Rows >= rows_valid give 0.  All 64 lanes must call.
+template <typename E, int D>
+__device__ __forceinline__ float resident_row_delta(const Resident<E, D>& dof, const typename Elem<E>::type* o_rows,
+                                                    int64_t o_stride, int rows_valid, int lane) {
+    using ET = typename Elem<E>::type;
+    constexpr int NJ = Resident<E, D>::NJ;
+    constexpr int EPC = 16 / Elem<E>::kBytes;
+    Resident<E, D> of;
+    load_resident<E, D>(of, o_rows, o_stride, rows_valid, lane);
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) {
+        // (plain conversions and fused multiply-adds: v_dot2_f32_bf16 gave wrong sums here)
+        const ET* a = reinterpret_cast<const ET*>(&of.c[j]);
+        const ET* d = reinterpret_cast<const ET*>(&dof.c[j]);
+#pragma unroll
+        for (int e = 0; e < EPC; e++) acc += Elem<E>::to_float(a[e]) * Elem<E>::to_float(d[e]);
+    }
+    return acc + __shfl_xor(acc, 32, 64);
+}
+
 // Store one output row from transposed accumulators: lane (n, h) holds, for every 32-wide block
 // db of the head dim, the 16 values of columns d = 32*db + 8*(r/4) + 4*h + r%4 of ITS row.
 // Each group of four consecutive r is four consecutive d.  fp32: one 16-byte store per group.  16-bit

@@ -47,7 +47,11 @@ struct BwdParams {
     const float* lse;
     const float* delta;
     const int32_t* lens;  // nullable
-    Strides3 sq, sk, sv, sdo, sdq, sdk, sdv;
+    // dQ that computes delta itself (chill_bwd_dq_delta): the forward's output, and where the rows of
+    // delta = rowsum(O * dO) go for the dK/dV launch that follows; both null otherwise
+    const void* o;
+    float* delta_out;
+    Strides3 sq, sk, sv, sdo, sdq, sdk, sdv, so;
     int64_t lse_b, lse_h;
     int64_t delta_b, delta_h;
     int64_t lens_stride;

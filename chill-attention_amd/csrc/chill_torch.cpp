@@ -35,9 +35,8 @@ struct EntryPoints {
     uint32_t abi_version;  // CHILL_ABI_VERSION of the header the table was filled against
     uint32_t bytes;        // sizeof(EntryPoints)
     decltype(&chill_fwd) fwd;
-    decltype(&chill_bwd_delta) delta;
+    decltype(&chill_bwd_dq_delta) dq_delta;
     decltype(&chill_bwd_dkdv) dkdv;
-    decltype(&chill_bwd_dq) dq;
     decltype(&chill_status_string) status_string;
 };
 
@@ -161,13 +160,13 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> backward_impl(const at::Tensor& q
     const int32_t B = (int32_t)q.size(0), H = (int32_t)q.size(1), H_kv = (int32_t)k.size(1), T = (int32_t)q.size(2),
                   D = (int32_t)q.size(3), dtype = dtype_code(q);
     void* stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    check(ep, "chill_bwd_delta", ep->delta(&to, &tdo, delta.data_ptr<float>(), delta_stride, B, H, T, D, dtype, stream));
+    // dQ first: it computes delta of its rows on the way and leaves it for dK/dV
+    check(ep, "chill_bwd_dq_delta",
+          ep->dq_delta(&tq, &tk, &tv, &to, &tdo, &tdq, lse.data_ptr<float>(), lse_stride, delta.data_ptr<float>(),
+                       delta_stride, lens_ptr, lens_stride, B, H, H_kv, T, D, dtype, (float)sm_scale, &desc, stream));
     check(ep, "chill_bwd_dkdv",
           ep->dkdv(&tq, &tk, &tv, &tdo, &tdk, &tdv, lse.data_ptr<float>(), lse_stride, delta.data_ptr<float>(),
                    delta_stride, lens_ptr, lens_stride, B, H, H_kv, T, D, dtype, (float)sm_scale, &desc, stream));
-    check(ep, "chill_bwd_dq",
-          ep->dq(&tq, &tk, &tv, &tdo, &tdq, lse.data_ptr<float>(), lse_stride, delta.data_ptr<float>(), delta_stride,
-                 lens_ptr, lens_stride, B, H, H_kv, T, D, dtype, (float)sm_scale, &desc, stream));
     return {dq, dk, dv};
 }
 
@@ -229,7 +228,7 @@ extern "C" int64_t chill_torch_register_entry_points(const void* table) {
     if (t.magic != kEntryPointsMagic || t.bytes != sizeof(EntryPoints)) return -1;
     if (t.abi_version != CHILL_ABI_VERSION) return -2;
     std::memcpy(&t, table, sizeof(EntryPoints));
-    if (!t.fwd || !t.delta || !t.dkdv || !t.dq || !t.status_string) return -1;
+    if (!t.fwd || !t.dq_delta || !t.dkdv || !t.status_string) return -1;
     std::lock_guard<std::mutex> lock(g_tables_mutex);
     g_tables.push_back(t);
     return (int64_t)g_tables.size() - 1;

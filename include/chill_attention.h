@@ -123,6 +123,22 @@ int chill_bwd_dq(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor
                  int32_t dtype, float sm_scale,
                  const ChillMaskDesc* mask, void* stream);
 
+/* dQ with the backward preprocessing fused into it: the launches of _chill_attn_bwd_precompute
+ * (utils.py:94-217, at chill.py:278-290) and of the dq branch of _chill_attn_bwd (chill_bwd_dq.py:15-397)
+ * in one.  Every workgroup computes delta = rowsum(O * dO) of its own query rows from the dO rows it
+ * loads anyway and the same rows of `o`, uses them, and WRITES them to `delta` (every row, zeros at and
+ * beyond lens[b]) for the chill_bwd_dkdv launch that must follow on the same stream.  One pass over O and
+ * one kernel boundary less than chill_bwd_delta + chill_bwd_dq; dq as from chill_bwd_dq up to the
+ * rounding of delta's sum (a different order of additions). */
+int chill_bwd_dq_delta(const ChillTensor4* q, const ChillTensor4* k, const ChillTensor4* v,
+                       const ChillTensor4* o, const ChillTensor4* d_o, const ChillTensor4* dq,
+                       const float* lse, const int64_t lse_stride[3],
+                       float* delta, const int64_t delta_stride[3],
+                       const int32_t* lens, int64_t lens_stride,
+                       int32_t B, int32_t H, int32_t H_kv, int32_t T, int32_t D,
+                       int32_t dtype, float sm_scale,
+                       const ChillMaskDesc* mask, void* stream);
+
 /* dK, dV: replaces the dkdv branch of _chill_attn_bwd (chill_bwd.py:130-167 ->
  * chill_bwd_dkdv.py:15-509), launched at chill.py:442.  One workgroup per (batch, kv head,
  * k-tile); the GQA group loop (chill_bwd_dkdv.py:156) runs inside it.  Every row of `dk` and `dv`
@@ -137,8 +153,8 @@ int chill_bwd_dkdv(const ChillTensor4* q, const ChillTensor4* k, const ChillTens
                    int32_t dtype, float sm_scale,
                    const ChillMaskDesc* mask, void* stream);
 
-/* The whole backward (delta, then dK/dV, then dQ, as chill_bwd_delta + chill_bwd_dkdv + chill_bwd_dq with
- * the same arguments) WITHOUT a delta workspace from the caller.  It has no counterpart in the
+/* The whole backward (dQ with delta on its way, then dK/dV: chill_bwd_dq_delta + chill_bwd_dkdv with the same
+ * arguments) WITHOUT a delta workspace from the caller.  It has no counterpart in the
  * reference: it is for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid it).  The fp32 delta rows live in an array inside the library,
  * CHILL_BWD_NOALLOC_MAX_ROWS floats (16 MiB) that every GPU the library runs on holds until the process

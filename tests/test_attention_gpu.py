@@ -647,6 +647,89 @@ def test_delta_kernel(D, dtype):
     np.testing.assert_allclose(delta.cpu().numpy(), want, atol=2e-5 * D, rtol=1e-5)
 
 
+# One shape per dQ kernel: (id, dtype, D, B, H, Hkv, T, mask, lens, (rows, waves, streamed) of the dQ row)
+DQ_DELTA_CASES = [
+    ("eight-waves", torch.bfloat16, 128, 2, 8, 8, 4500, ("CausalChillMask", ()), (4500, 1000), (256, 8, 64)),
+    ("four-waves-gqa-f16", torch.float16, 64, 2, 8, 2, 1100, ("PrefixLMChillMask", (100,)), None, (128, 4, 64)),
+    ("four-waves-window", torch.bfloat16, 128, 1, 16, 16, 2100, ("SlidingWindowChillMask", (100, 30)), (1999,), (128, 4, 64)),
+    ("registers-128", torch.bfloat16, 128, 1, 16, 8, 8200, ("CausalChillMask", ()), (8111,), (256, 4, 32)),
+    ("registers-256-f16", torch.float16, 256, 1, 8, 8, 1030, ("FullChillMask", ()), (700,), (128, 4, 32)),
+    ("split-f32-256", torch.float32, 256, 1, 4, 2, 530, ("CausalChillMask", ()), (333,), None),
+    ("f32-64", torch.float32, 64, 2, 8, 8, 1500, ("ChunkwiseChillMask", (64, 2)), (1500, 65), (128, 4, 32)),
+    ("small-launch", torch.bfloat16, 64, 1, 2, 1, 300, ("CausalChillMask", ()), (129,), (32, 4, 32)),
+    ("small-launch-f32", torch.float32, 32, 1, 3, 3, 257, ("FullChillMask", ()), None, (32, 4, 32)),
+]
+
+
+@pytest.mark.parametrize("case", DQ_DELTA_CASES, ids=lambda c: c[0])
+def test_dq_computes_delta_on_its_way(case):
+    """chill_bwd_dq_delta (what the operator's backward launches before dK/dV) through the C ABI, on one shape per dQ
+    kernel (route asserted from the tile table): the delta rows it leaves behind equal the closed form rowsum(O * dO)
+    in fp64 (utils.py:190) on every row below lens[b] and are finite on every other row (the buffer starts as NaN),
+    and its dQ equals what chill_bwd_dq computes from chill_bwd_delta's rows, up to the rounding of a sum of D
+    products taken in another order."""
+    import ctypes
+
+    _, dtype, D, B, H, Hkv, T, m, lens, route = case
+    mask = make_mask(m)
+    if route is not None:
+        cfg = tile_config(mask, D, dtype, _lib.PASS_DQ, seq_len=T, batch_heads=B * H)
+        assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == route, f"served by {cfg}"
+    torch.manual_seed(stable_seed(case[0]))
+    q, k, v = (make_qkv((B, h, T, D), dtype, False) for h in (H, Hkv, Hkv))
+    do = torch.randn(B, T, H, D, device=DEV, dtype=dtype).transpose(1, 2)  # a strided view
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    o, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens_t, return_lse=True)
+    code = {torch.float32: _lib.F32, torch.float16: _lib.F16, torch.bfloat16: _lib.BF16}[dtype]
+    desc = mask.descriptor()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    lens_p = (None, 0) if lens_t is None else (ctypes.c_void_p(lens_t.data_ptr()), lens_t.stride(0))
+    t = {n: _lib.tensor4(x) for n, x in (("q", q), ("k", k), ("v", v), ("o", o), ("do", do))}
+    r = lambda n: ctypes.byref(t[n])  # noqa: E731
+    lse_p, s_lse = ctypes.c_void_p(lse.data_ptr()), _lib.strides3(lse)
+    sm_scale = D ** -0.5
+    L = _lib.lib
+    # the two launches of the reference's structure
+    delta = torch.empty(B, H, T, dtype=torch.float32, device=DEV)
+    want = torch.full_like(q, float("nan"))
+    tw = _lib.tensor4(want)
+    _lib.check("chill_bwd_delta", L.chill_bwd_delta(r("o"), r("do"), ctypes.c_void_p(delta.data_ptr()), _lib.strides3(delta),
+                                                    B, H, T, D, code, stream))
+    _lib.check("chill_bwd_dq", L.chill_bwd_dq(r("q"), r("k"), r("v"), r("do"), ctypes.byref(tw), lse_p, s_lse,
+                                              ctypes.c_void_p(delta.data_ptr()), _lib.strides3(delta), *lens_p, B, H, Hkv, T, D,
+                                              code, sm_scale, ctypes.byref(desc), stream))
+    # the fused one, into a buffer of NaNs
+    delta2 = torch.full((B, H, T), float("nan"), dtype=torch.float32, device=DEV)
+    got = torch.full_like(q, float("nan"))
+    tg = _lib.tensor4(got)
+    _lib.check("chill_bwd_dq_delta", L.chill_bwd_dq_delta(
+        r("q"), r("k"), r("v"), r("o"), r("do"), ctypes.byref(tg), lse_p, s_lse, ctypes.c_void_p(delta2.data_ptr()),
+        _lib.strides3(delta2), *lens_p, B, H, Hkv, T, D, code, sm_scale, ctypes.byref(desc), stream))
+    torch.cuda.synchronize()
+    assert torch.isfinite(delta2).all(), "a row of delta was left unwritten"
+    closed = orc.delta(o.double().cpu().numpy(), do.double().cpu().numpy())
+    for b in range(B):
+        n = T if lens is None else lens[b]
+        np.testing.assert_allclose(delta2[b, :, :n].cpu().numpy(), closed[b, :, :n], atol=2e-5 * D, rtol=1e-5)
+    assert torch.isfinite(got).all()
+    tol = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}[dtype]
+    torch.testing.assert_close(got.float(), want.float(), atol=tol, rtol=tol)
+    # and dK/dV from the rows the fused launch left behind equal dK/dV from chill_bwd_delta's rows to the same bar
+    grads = []
+    for rows in (delta, delta2):
+        dk, dv = torch.full_like(k, float("nan")), torch.full_like(v, float("nan"))
+        tdk, tdv = _lib.tensor4(dk), _lib.tensor4(dv)
+        _lib.check("chill_bwd_dkdv", L.chill_bwd_dkdv(
+            r("q"), r("k"), r("v"), r("do"), ctypes.byref(tdk), ctypes.byref(tdv), lse_p, s_lse,
+            ctypes.c_void_p(rows.data_ptr()), _lib.strides3(rows), *lens_p, B, H, Hkv, T, D, code, sm_scale,
+            ctypes.byref(desc), stream))
+        grads.append((dk, dv))
+    torch.cuda.synchronize()
+    for a, b_ in zip(grads[0], grads[1]):
+        assert torch.isfinite(b_).all()
+        torch.testing.assert_close(b_.float(), a.float(), atol=tol, rtol=tol)
+
+
 @pytest.mark.parametrize("T,D,dtype", [(70001, 64, torch.float16), (100003, 128, torch.bfloat16)])
 def test_long_sequences(T, D, dtype):
     """Sequences far beyond the BASELINE sizes, of a length no tile divides (row offsets past 2^24 elements):

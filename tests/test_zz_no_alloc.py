@@ -1,5 +1,5 @@
-"""The backward entry point that takes no delta workspace (chill_bwd_noalloc) against the three entry
-points it stands for (chill_bwd_delta + chill_bwd_dkdv + chill_bwd_dq with a caller-owned delta), through
+"""The backward entry point that takes no delta workspace (chill_bwd_noalloc) against the two entry
+points it stands for (chill_bwd_dq_delta + chill_bwd_dkdv with a caller-owned delta), through
 the C ABI: two calls in a row, the second with a smaller input, so that what the first call left in the
 library's array cannot pass for the second call's rows.  Integer-exact comparison: the same kernels run on
 the same values."""
@@ -41,12 +41,11 @@ def backward_both_ways(mask, B, H, Hkv, T, D, dtype, lens, seed):
     delta = torch.empty(B, H, T, dtype=torch.float32, device=DEV)
     delta_p, s_delta = ctypes.c_void_p(delta.data_ptr()), _lib.strides3(delta)
     L = _lib.lib
-    _lib.check("chill_bwd_delta", L.chill_bwd_delta(r("o"), r("do"), delta_p, s_delta, B, H, T, D, code, stream))
+    _lib.check("chill_bwd_dq_delta", L.chill_bwd_dq_delta(r("q"), r("k"), r("v"), r("o"), r("do"), ctypes.byref(tw["dq"]), lse_p, s_lse,
+                                                          delta_p, s_delta, *lens_p, B, H, Hkv, T, D, code, sm_scale, ctypes.byref(desc), stream))
     _lib.check("chill_bwd_dkdv", L.chill_bwd_dkdv(r("q"), r("k"), r("v"), r("do"), ctypes.byref(tw["dk"]), ctypes.byref(tw["dv"]),
                                                   lse_p, s_lse, delta_p, s_delta, *lens_p, B, H, Hkv, T, D, code, sm_scale,
                                                   ctypes.byref(desc), stream))
-    _lib.check("chill_bwd_dq", L.chill_bwd_dq(r("q"), r("k"), r("v"), r("do"), ctypes.byref(tw["dq"]), lse_p, s_lse, delta_p,
-                                              s_delta, *lens_p, B, H, Hkv, T, D, code, sm_scale, ctypes.byref(desc), stream))
     # the entry point without a workspace
     got, tg = outputs()
     _lib.check("chill_bwd_noalloc", L.chill_bwd_noalloc(
@@ -76,7 +75,7 @@ def test_backward_without_workspace_equals_backward_with_one():
 def test_captured_in_a_hip_graph_after_a_first_call():
     """chill_bwd_noalloc recorded into a HIP graph (its first call on the device has happened before, outside the
     capture, as the header asks: that call looks the array's address up): every replay, with new contents in the
-    static inputs and eager work and synchronisations in between, equals the three entry points run eagerly."""
+    static inputs and eager work and synchronisations in between, equals the operator's own backward run eagerly."""
     mask = ca.ChunkwiseChillMask(40, 1)
     B, H, Hkv, T, D, dtype = 2, 4, 2, 300, 128, torch.bfloat16
     backward_both_ways(mask, 1, 2, 2, 64, 64, dtype, None, seed=5)  # the first call on this device, if none was made yet
