@@ -45,9 +45,6 @@ CANDIDATES = [
                    "CHILL_TUNE_DQ_STREAMED": 64, "CHILL_TUNE_FWD_STAGES": 2, "CHILL_TUNE_DQ_STAGES": 2}),
     ("w4_s32_n3", {"CHILL_TUNE_FWD_WAVES": 4, "CHILL_TUNE_DQ_WAVES": 4, "CHILL_TUNE_FWD_STREAMED": 32,
                    "CHILL_TUNE_DQ_STREAMED": 32, "CHILL_TUNE_FWD_STAGES": 3, "CHILL_TUNE_DQ_STAGES": 3}),
-    # dK/dV with 64 key rows per wave, K in registers and the accumulators in hand-managed accumulation
-    # registers (head dims 64 and 128): as fast as the shipped paired kernel, not faster
-    ("dkdv_r64", {"CHILL_TUNE_DKDV_R64": 1, "__flags__": "-mllvm -amdgpu-spill-vgpr-to-agpr=0"}),
 ]
 
 _HIPFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Wno-unused-value",
@@ -98,13 +95,13 @@ def kernel_resources(elem: str = "bf16", dim: int = 128, macros: dict | None = N
 
 def check_hand_managed_registers(macros: dict | None = None) -> None:
     """Raise RuntimeError unless, in every kernel that names accumulation registers itself (16-bit inputs:
-    the three kernels of head dim 256, dK/dV with register-resident K at head dim 128), the compiler stays
+    the three kernels of head dim 256, dK/dV with register-resident K at head dims 64 and 128, dQ with register-resident Q and dO at head dim 128), the compiler stays
     below the registers the kernel names.  Spilled registers are accepted only where the compiler touches
     no accumulation register at all (they are in scratch memory then, not parked in accumulation
     registers).  The check reads the assembly hipcc writes for the given build (``macros`` as for the
     library build); it covers register overlap and spills, nothing else.  Part of every build of the library."""
     for elem in ("bf16", "f16"):
-        for dim in (256, 128):
+        for dim in (256, 128, 64):
             rows = hand_managed_registers(elem, dim, macros)
             if not rows:
                 raise RuntimeError(f"no hand-managed kernel found for {elem} head dim {dim}")

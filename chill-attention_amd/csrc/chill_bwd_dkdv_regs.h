@@ -14,12 +14,12 @@
 // CB = 1, D = 256 (512-byte rows) is the shipped dK/dV kernel of that shape: 2 x 8 accumulator blocks
 // are exactly the 256 accumulation registers, which the compiler cannot keep there by itself (its
 // version of this kernel spills 2400 registers to scratch and runs 40x slower).
-// CB = 2, D = 128 is the dK/dV kernel of long sequences at that head dim (chill_tiles.h: dkdv_takes_regs):
-// every streamed operand fetched from LDS feeds two MFMAs and K is never re-read, 76 LDS reads per 64
-// MFMAs where the paired kernel needs 146.  Its runs of predicate-free tiles go through a generated,
-// hazard-checked loop (gen_bwd_loop.py -> chill_bwd_loop.inc); with the compiler's schedule the shape was
-// no faster than the paired kernel (a lone wave hides its vector work only behind its own MFMAs).  The
-// same shape at D = 64 remains a sweep candidate (-DCHILL_TUNE_DKDV_R64=1, compiler-scheduled).
+// CB = 2, D = 64 / 128 is the dK/dV kernel of long sequences at those head dims (chill_tiles.h:
+// dkdv_takes_regs): every streamed operand fetched from LDS feeds two MFMAs and K is never re-read, at
+// D = 128 76 LDS reads per 64 MFMAs where the paired kernel needs 146.  Its runs of predicate-free tiles
+// go through a generated, hazard-checked loop (gen_bwd_loop.py -> chill_bwd_loop.inc); with the
+// compiler's schedule the shape was no faster than the paired kernel (a lone wave hides its vector work
+// only behind its own MFMAs).
 //
 // Every translation unit that instantiates this kernel is checked (tests/test_abi.py) for the
 // compiler keeping out of the accumulation registers the kernel names itself.
@@ -38,7 +38,7 @@ namespace chill {
 // stored times -sm_scale.
 template <typename E, int D, int CB, int NS>
 constexpr bool dkdv_has_generated_loop() {
-    return Elem<E>::k16 && D == 128 && CB == 2 && NS == 4;
+    return Elem<E>::k16 && (D == 128 || D == 64) && CB == 2 && NS == 4;
 }
 
 template <typename E, int D, int MASK, int CB, int NS>
@@ -177,9 +177,11 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
     // What the generated loop takes besides K: per-lane LDS addresses with everything wave-dependent folded in
     // (an LDS read of the loop is one of these registers plus a constant), the per-lane offsets of the tile
     // loads, and scalars.
-    [[maybe_unused]] unsigned a_qrow[NJ], a_qtr[DB][2], a_vrow[NJ], a_vec = 0;
+    // (rows of 128 bytes: the two 16-row halves of a tile have transposed-operand addresses of their own)
+    constexpr int NTR = OperandOffsets<E, D>::NS_TR;
+    [[maybe_unused]] unsigned a_qrow[NJ], a_qtr[DB][NTR][2], a_vrow[NJ], a_vec = 0;
     if constexpr (kGen) {
-        static_assert(L::kBlockAffine && OperandOffsets<E, D>::kHalfAffine, "rows of 256 bytes");
+        static_assert(L::kBlockAffine, "rows of 128 bytes and more");
         const unsigned ring = lds_address(smem + V_BYTES), vtile = lds_address(smem) + CB * wave * L::BLOCK_BYTES;
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
@@ -189,7 +191,9 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
-            for (int w = 0; w < 2; w++) a_qtr[db][w] = ring + ofs.tr[db][0][w];
+            for (int sx = 0; sx < NTR; sx++)
+#pragma unroll
+                for (int w = 0; w < 2; w++) a_qtr[db][sx][w] = ring + ofs.tr[db][sx][w];
         a_vec = ring + 2 * TILE_BYTES + 16 * h;
     }
     // first tile of iteration `it` and its pointers (the generated loop moves them on by itself)
@@ -237,21 +241,37 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
                 const unsigned vecwave = uniform(wave == NW - 1 ? 1u : 0u);
                 const unsigned lane4 = lane * 4;
                 const float scale_s = uniform(p.scale_log2);
-#define CHILL_DKDV_LOOP_ARGS                                                                                          \
+#define CHILL_DKDV_LOOP_ARGS_128                                                                                      \
     cnt, tok, qp, dop, lsep, delp, kf[0].c[0], kf[0].c[1], kf[0].c[2], kf[0].c[3], kf[0].c[4], kf[0].c[5], kf[0].c[6], \
         kf[0].c[7], kf[1].c[0], kf[1].c[1], kf[1].c[2], kf[1].c[3], kf[1].c[4], kf[1].c[5], kf[1].c[6], kf[1].c[7],     \
-        a_qrow[0], a_qrow[1], a_qrow[2], a_qrow[3], a_qrow[4], a_qrow[5], a_qrow[6], a_qrow[7], a_qtr[0][0],            \
-        a_qtr[0][1], a_qtr[1][0], a_qtr[1][1], a_qtr[2][0], a_qtr[2][1], a_qtr[3][0], a_qtr[3][1], a_vrow[0],           \
-        a_vrow[1], a_vrow[2], a_vrow[3], a_vrow[4], a_vrow[5], a_vrow[6], a_vrow[7], a_vec, load_q.goff[0],             \
-        load_q.goff[1], load_do.goff[0], load_do.goff[1], lane4, scale_s, dmabase, vecdma, qstep, dostep, vecwave, st0, tailn
+        a_qrow[0], a_qrow[1], a_qrow[2], a_qrow[3], a_qrow[4], a_qrow[5], a_qrow[6], a_qrow[7], a_qtr[0][0][0],         \
+        a_qtr[0][0][1], a_qtr[1][0][0], a_qtr[1][0][1], a_qtr[2][0][0], a_qtr[2][0][1], a_qtr[3][0][0], a_qtr[3][0][1], \
+        a_vrow[0], a_vrow[1], a_vrow[2], a_vrow[3], a_vrow[4], a_vrow[5], a_vrow[6], a_vrow[7], a_vec, load_q.goff[0],  \
+        load_q.goff[1], load_do.goff[0], load_do.goff[1], lane4, scale_s, dmabase, vecdma, qstep, dostep, vecwave, st0, \
+        tailn
+#define CHILL_DKDV_LOOP_ARGS_64                                                                                       \
+    cnt, tok, qp, dop, lsep, delp, kf[0].c[0], kf[0].c[1], kf[0].c[2], kf[0].c[3], kf[1].c[0], kf[1].c[1], kf[1].c[2], \
+        kf[1].c[3], a_qrow[0], a_qrow[1], a_qrow[2], a_qrow[3], a_qtr[0][0][0], a_qtr[0][0][1], a_qtr[0][1][0],         \
+        a_qtr[0][1][1], a_qtr[1][0][0], a_qtr[1][0][1], a_qtr[1][1][0], a_qtr[1][1][1], a_vrow[0], a_vrow[1],           \
+        a_vrow[2], a_vrow[3], a_vec, load_q.goff[0], load_do.goff[0], lane4, scale_s, dmabase, vecdma, qstep, dostep,   \
+        vecwave, st0, tailn
 #define CHILL_DKDV_LOOP_CALL(loop, ...) loop(__VA_ARGS__)
-                if constexpr (std::is_same<E, bf16_t>::value) {
-                    CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_BF16_128, CHILL_DKDV_LOOP_ARGS);
+                if constexpr (D == 128) {
+                    if constexpr (std::is_same<E, bf16_t>::value) {
+                        CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_BF16_128, CHILL_DKDV_LOOP_ARGS_128);
+                    } else {
+                        CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_F16_128, CHILL_DKDV_LOOP_ARGS_128);
+                    }
                 } else {
-                    CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_F16_128, CHILL_DKDV_LOOP_ARGS);
+                    if constexpr (std::is_same<E, bf16_t>::value) {
+                        CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_BF16_64, CHILL_DKDV_LOOP_ARGS_64);
+                    } else {
+                        CHILL_DKDV_LOOP_CALL(CHILL_DKDV_LOOP_F16_64, CHILL_DKDV_LOOP_ARGS_64);
+                    }
                 }
 #undef CHILL_DKDV_LOOP_CALL
-#undef CHILL_DKDV_LOOP_ARGS
+#undef CHILL_DKDV_LOOP_ARGS_128
+#undef CHILL_DKDV_LOOP_ARGS_64
                 st_cur = (st_cur + n_run) % NS;
                 st_issue = (st_issue + n_run) % NS;
                 tile = t_next + n_run - 1;

@@ -36,9 +36,6 @@
 #ifndef CHILL_TUNE_DKDV_WAVES
 #define CHILL_TUNE_DKDV_WAVES 0
 #endif
-#ifndef CHILL_TUNE_DKDV_R64
-#define CHILL_TUNE_DKDV_R64 0
-#endif
 
 // 1: the 8-wave forward of 16-bit inputs at head dim 128 streams 64-key tiles through four stages,
 // the shape fwd_q_tile_fast and its generated loop are written for; 0: the shape before it (128-key
@@ -266,38 +263,40 @@ constexpr int dkdv_split_lds_bytes(int D, int dtype) {
 
 // dK/dV with hand-managed accumulation registers (dkdv_regs_kernel, 16-bit inputs): 4 waves, K in
 // registers, V in LDS, 32-row Q / dO tiles in a ring.  blocks = 32-key blocks per wave:
-//   * head dim 256: one block per wave (128 key rows per workgroup), two ring stages: the shipped
+//   * head dim 256: one block per wave (128 key rows per workgroup), two ring stages: the only
 //     kernel of that shape;
-//   * head dim 64 / 128 with -DCHILL_TUNE_DKDV_R64=1: two blocks per wave (256 key rows), four stages:
-//     a sweep candidate.
+//   * head dims 64 and 128: two blocks per wave (256 key rows), four stages, beside the paired kernel
+//     (dkdv_regs_is_optional below).
 constexpr int dkdv_regs_blocks(int D, int dtype) {
     if (dtype == CHILL_F32) return 0;
     if (D == 256) return 1;
-    if (CHILL_TUNE_DKDV_R64 && (D == 64 || D == 128)) return 2;
     return 0;
 }
 constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
-// 16-bit inputs at head dim 128 have both kernels: the paired one, and dkdv_regs_kernel with two blocks per wave,
+// 16-bit inputs at head dims 64 and 128 have both kernels: the paired one, and dkdv_regs_kernel with two blocks per wave,
 // whose runs of predicate-free tiles go through a generated loop (gen_bwd_loop.py).  The latter owns its CU (130 KiB of
 // LDS, 512 registers per wave) and pays more before and after its loop (K into registers, V negated in LDS, no second
 // workgroup to hide behind): it is taken for long sequences on a grid of at least two workgroups per CU, and of
 // the banded masks only for those named below.  Measured on dK/dV alone, against the paired kernel:
 // causal B8 H16 T8192 3.63 / 4.06 ms, B16 H16 T4096 2.18 / 2.27, B2 H8 T8192 0.547 / 0.591, full mask fp16 B4 H16
 // T4096 0.98 / 1.16, prefix-LM B4 H16 T8192 1.91 / 2.16; but causal B1 H8 T8192 0.368 / 0.318, B4 H16 T2048
-// 0.227 / 0.197, sliding window 512 at T8192 0.65 / 0.49.
+// 0.227 / 0.197, sliding window 512 at T8192 0.65 / 0.49.  At head dim 64 (against the 4-wave kernel that runs three
+// to a CU): causal B8 H16 T4096 0.73 / 0.77, B4 H32 T8192 2.12 / 2.42, B2 H8 T8192 0.31 / 0.36, B1 H32 T16384 1.99 / 2.35,
+// full mask B4 H16 T4096 0.56 / 0.73, prefix-LM B4 H32 T8192 2.12 / 2.45.
 constexpr int kDkdvRegsBlocks128 = 2;
 constexpr int kDkdvRegsMinSequence = 4096;
 constexpr int kDkdvRegsMinWorkgroups = 2 * 256;
-constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && D == 128 && !CHILL_TUNE_DKDV_R64; }
+constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && (D == 128 || D == 64); }
 // Banded masks take it only when a wave's 64 key rows lie in one chunk, so that its tiles are all predicate-free
 // and all alike: chunkwise masks whose chunk size is a multiple of 64 (`mask_arg0` = the mask's first argument;
 // measured at head dim 128, T = 8192 and 16384: chunks of 64 / 128 / 256 / 1024 rows -5 / -8 / -13 / -16 %, chunks
-// of 96 rows +13 %, sliding windows of 64 .. 512 rows +32 .. +60 %, of 1024 rows and more +-1 %).
-constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0) {
-    return mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0;
+// of 96 rows +13 %, sliding windows of 64 .. 512 rows +32 .. +60 %, of 1024 rows and more +-1 %; at head dim 64,
+// where a tile is half the work, chunks of 64 rows +30 .. +68 %, of 128 rows +-1 %, of 1024 rows -17 %: from 256 rows on).
+constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0, int D) {
+    return mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0 && (D >= 128 || mask_arg0 >= 256);
 }
-constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, long long batch_kv_heads, int T) {
-    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0)) && T >= kDkdvRegsMinSequence &&
+constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, int D, long long batch_kv_heads, int T) {
+    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, D)) && T >= kDkdvRegsMinSequence &&
            batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >= kDkdvRegsMinWorkgroups;
 }
 
@@ -353,8 +352,8 @@ inline int tile_config(int mask_id, long long mask_arg0, int D, int dtype, int p
             }
             // (the row of long sequences on a full chip: the generated loop where there is one)
             *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T),
-                                    T == kLongSequence ? (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0))
-                                                       : dkdv_takes_regs(mask_id, mask_arg0, batch_heads, T));
+                                    T == kLongSequence ? (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, D))
+                                                       : dkdv_takes_regs(mask_id, mask_arg0, D, batch_heads, T));
             return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }

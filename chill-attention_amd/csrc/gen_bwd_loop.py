@@ -49,8 +49,21 @@ SPECIAL_CLOBBERS = ["vcc", "scc", "m0"]
 
 
 class Config:
-    def __init__(self, elem: str, D: int = 128, units: int = 10, barrier_slot: int = 56, split_a: bool = True):
-        assert elem in ("bf16", "f16") and D == 128
+    # Slot windows of the vector work, per head dim: exponentials of block 0, of the two halves of block 1
+    # (split_a) or of everything (not split_a), products and packs of entries 0..7 and 8..15, the slot the
+    # next iteration's barrier stands in front of, the last slot that carries tile loads.
+    WINDOWS = {
+        128: dict(e0=(10, 23), e1a=(24, 31), e1b=(32, 39), e=(18, 39), g0=(40, 45), p0=(44, 47), g1=(46, 51),
+                  p1=(52, 55), barrier=56, dma=15),
+        64: dict(e0=(6, 11), e1a=(12, 15), e1b=(16, 19), e=(9, 19), g0=(20, 22), p0=(22, 23), g1=(23, 25),
+                 p1=(26, 27), barrier=28, dma=7),
+    }
+
+    def __init__(self, elem: str, D: int = 128, units: int = 10, barrier_slot: int = None, split_a: bool = True):
+        assert elem in ("bf16", "f16") and D in self.WINDOWS
+        self.win = self.WINDOWS[D]
+        if barrier_slot is None:
+            barrier_slot = self.win["barrier"]
         self.elem, self.D = elem, D
         self.CB, self.NSTG, self.NW = 2, 4, 4
         self.NJ = D // 16                 # MFMAs of a 32 x 32 product over the head dim
@@ -74,7 +87,11 @@ class Config:
         self.mfma = "v_mfma_f32_32x32x16_" + elem
         self.cvt = "v_cvt_pk_bf16_f32" if elem == "bf16" else "v_cvt_pk_f16_f32"
         self.name = f"CHILL_DKDV_LOOP_{elem.upper()}_{D}"
-        self.loads_per_tile = 4           # per wave: two slabs of Q, two of dO (the wave with the vectors: two more)
+        # rows 16 apart share the swizzle key of their chunks only in rows of 256 bytes and more: below that the
+        # transposed operands of the two 16-row halves of a tile have per-lane addresses of their own
+        self.half_affine = self.row_bytes >= 256
+        self.slabs = self.tile // (self.NW * 1024)   # 1 KiB slabs of a tile that one wave loads: 2, or 1 at head dim 64
+        self.loads_per_tile = 2 * self.slabs         # per wave: Q and dO (the wave with the vectors: two more)
 
     def dv(self, c, db):
         return AGPR + 16 * (c * self.DB + db)
@@ -131,7 +148,7 @@ def dma_ops(c: Config, st: Stream, tgt: int):
     ops = []
     base = tgt * c.stage
     for name, off in (("q", 0), ("do", c.tile)):
-        for i in range(2):
+        for i in range(c.slabs):
             def load(name=name, off=off, i=i):
                 A(f"s_add_u32 m0, %[dmabase], {base + off + i * c.NW * 1024}", "salu")
                 A("s_nop 0", "nop")
@@ -250,11 +267,12 @@ class Iteration:
         for sx in range(2):
             for db in range(c.DB):
                 queue.append((("qt", sx, db), 0))
-        E_LO, E_HI = 18, 39          # slots of the exponentials
-        G0_LO, G0_HI = 40, 45        # products of entries 0..7
-        P0_LO, P0_HI = 44, 47        # their pack (PB[0:3] is free once slot 39 has been issued)
-        G1_LO, G1_HI = 46, 51
-        P1_LO, P1_HI = 52, 55
+        w = c.win
+        E_LO, E_HI = w["e"]          # slots of the exponentials
+        G0_LO, G0_HI = w["g0"]       # products of entries 0..7
+        P0_LO, P0_HI = w["p0"]       # their pack (PB[0:3] is free once the dV^T MFMAs of the first half have been issued)
+        G1_LO, G1_HI = w["g1"]
+        P1_LO, P1_HI = w["p1"]
         if with_prefetch:
             for g in range(4):
                 queue.append((("nlse", g), E_HI + 1))
@@ -273,9 +291,10 @@ class Iteration:
             if kind == "v":
                 return [(f"ds_read_b128 {vr(u, 4)}, %[vrow{key[2]}] offset:{key[1] * c.tile}", rng(u, 4))]
             if kind in ("dot", "qt"):
-                off = s * c.stage + (c.tile if kind == "dot" else 0) + key[1] * 16 * c.row_bytes
-                return [(f"ds_read_b64_tr_b16 {vr(u, 2)}, %[qtr{key[2]}_0] offset:{off}", rng(u, 2)),
-                        (f"ds_read_b64_tr_b16 {vr(u + 2, 2)}, %[qtr{key[2]}_1] offset:{off}", rng(u + 2, 2))]
+                off = s * c.stage + (c.tile if kind == "dot" else 0) + (key[1] * 16 * c.row_bytes if c.half_affine else 0)
+                at = f"qtr{key[2]}" if c.half_affine else f"qtr{key[2]}_{key[1]}"
+                return [(f"ds_read_b64_tr_b16 {vr(u, 2)}, %[{at}_0] offset:{off}", rng(u, 2)),
+                        (f"ds_read_b64_tr_b16 {vr(u + 2, 2)}, %[{at}_1] offset:{off}", rng(u + 2, 2))]
             if kind == "nq":
                 return [(f"ds_read_b128 {vr(u, 4)}, %[qrow{key[1]}] offset:{nxt * c.stage}", rng(u, 4))]
             if kind == "nlse":
@@ -296,9 +315,9 @@ class Iteration:
             for t, lst in enumerate(deal(ops, lo, hi, NS)):
                 valu[t] += lst
         if c.split_a:
-            place(softmax_pairs(c, st, 0, range(0, 8)), 10, 23)
-            place(softmax_pairs(c, st, 1, range(0, 4)), 24, 31)
-            place(softmax_pairs(c, st, 1, range(4, 8)), 32, E_HI)
+            place(softmax_pairs(c, st, 0, range(0, 8)), *w["e0"])
+            place(softmax_pairs(c, st, 1, range(0, 4)), *w["e1a"])
+            place(softmax_pairs(c, st, 1, range(4, 8)), *w["e1b"])
         else:
             e_ops = []
             for half in (range(0, 4), range(4, 8)):
@@ -310,7 +329,7 @@ class Iteration:
         place(product_ops(c, st, 0, range(8, 16)) + product_ops(c, st, 1, range(8, 16)), G1_LO, G1_HI)
         place(pack_ops(c, st, 0, range(4, 8)) + pack_ops(c, st, 1, range(4, 8)), P1_LO, P1_HI)
         if with_dma and "dma" not in ABLATE:
-            scalar = deal(dma_ops(c, st, tgt), 0, 15, NS)
+            scalar = deal(dma_ops(c, st, tgt), 0, w["dma"], NS)
         elif "dma" not in ABLATE:
             # (the vector instructions behind the score MFMAs count on the issue slots the tile loads take)
             pads = []
@@ -319,7 +338,7 @@ class Iteration:
                 op()
                 n_ins = len(count.ins) - before
                 pads.append(lambda n_ins=n_ins: st.add(f"s_nop {n_ins - 1}", "nop", nops=n_ins))
-            scalar = deal(pads, 0, 15, NS)
+            scalar = deal(pads, 0, w["dma"], NS)
         else:
             scalar = [[] for _ in range(NS)]
 
@@ -548,11 +567,12 @@ def operand_lists(c: Config):
     for j in range(c.NJ):
         ins.append((f"qrow{j}", "v"))
     for db in range(c.DB):
-        for w in range(2):
-            ins.append((f"qtr{db}_{w}", "v"))
+        for sx in range(1 if c.half_affine else 2):
+            for w in range(2):
+                ins.append((f"qtr{db}_{w}" if c.half_affine else f"qtr{db}_{sx}_{w}", "v"))
     for j in range(c.NJ):
         ins.append((f"vrow{j}", "v"))
-    for n in ("vec", "gq0", "gq1", "gdo0", "gdo1", "lane4"):
+    for n in ["vec"] + [f"g{t}{i}" for t in ("q", "do") for i in range(c.slabs)] + ["lane4"]:
         ins.append((n, "v"))
     for n in ("scale", "dmabase", "vecdma", "qstep", "dostep", "vecwave", "st0", "tailn"):
         ins.append((n, "s"))
@@ -597,8 +617,9 @@ def main():
         if ABLATE:
             out.write("#ifndef CHILL_TIMING_EXPERIMENT\n#error \"a loop with parts left out (--ablate): timing experiments only\"\n#endif\n\n")
         kw = {k: v for k, v in (("barrier_slot", args.barrier_slot), ("units", args.units), ("split_a", args.split_a)) if v is not None}
-        for c in (Config("bf16", **kw), Config("f16", **kw)):
-            emit_macro(c, out)
+        for D in (128, 64):
+            for c in (Config("bf16", D, **kw), Config("f16", D, **kw)):
+                emit_macro(c, out)
     return 0
 
 

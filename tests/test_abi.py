@@ -138,10 +138,12 @@ def test_tile_table():
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
     assert _lib.lib.chill_tile_config_for_shape(1, 128, _lib.BF16, 0, 1, 0, (ctypes.c_int32 * 4)()) == -8
-    # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU
-    for D, rows, waves in ((64, 64, 4), (32, 64, 4)):
-        c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV)
+    # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU (at head dim 64
+    # for short sequences, small grids and banded masks; long sequences: K in registers, below)
+    for D, T, rows, waves in ((64, 4095, 64, 4), (32, None, 64, 4), (32, 8192, 64, 4)):
+        c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=1 << 12)
         assert (c["rows"], c["waves"]) == (rows, waves), (D, c)
+    assert tile_config(window, 64, torch.bfloat16, _lib.PASS_DKDV)["rows"] == 64
     # dQ at 16-bit head dim 128 from 8192 keys on, full grids, masks that are not banded: Q and dO in registers
     regs2 = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 4 * 2 * 32 * 256}
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_DQ) == regs2
@@ -174,7 +176,17 @@ def test_tile_table():
     assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, None) == -1
     desc.nargs = 1
     assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == -4
-    assert 2 * tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV)["lds_bytes"] <= 160 * 1024
+    # the same kernel at head dim 64 (rows of 128 bytes), for the same launches; of the chunkwise masks only chunks of
+    # 256 rows and more
+    regs64 = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 256 * 128 + 4 * (2 * 32 * 128 + 2 * 32 * 4)}
+    assert tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV) == regs64
+    assert tile_config(ca.PrefixLMChillMask(1024), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
+    assert tile_config(ca.ChunkwiseChillMask(256, 1), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
+    for mask, T, bh in ((causal, 4096, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64), (ca.ChunkwiseChillMask(64, 4), 8192, 64),
+                        (window, 8192, 128)):
+        c = tile_config(mask, 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
+        assert (c["rows"], c["waves"], c["streamed"]) == (64, 4, 64), (mask, T, bh, c)
+    assert 2 * tile_config(window, 64, torch.bfloat16, _lib.PASS_DKDV)["lds_bytes"] <= 160 * 1024
     tq, tk, waves = _get_default_config_fwd(128, torch.bfloat16)
     assert tq == 32 * waves and tk % 32 == 0
     (dq_q, dq_k, _), (dk_q, dk_k, _) = _get_default_config_bwd(128, torch.bfloat16)
@@ -246,7 +258,7 @@ def test_tile_sweep_candidates():
     names = [n for n, _ in tune.CANDIDATES]
     assert len(set(names)) == len(names) and tune.CANDIDATES[0][1] == {}
     allowed = {"CHILL_TUNE_FWD_WAVES", "CHILL_TUNE_FWD_STREAMED", "CHILL_TUNE_FWD_STAGES", "CHILL_TUNE_DQ_WAVES",
-               "CHILL_TUNE_DQ_STREAMED", "CHILL_TUNE_DQ_STAGES", "CHILL_TUNE_DKDV_WAVES", "CHILL_TUNE_DKDV_R64", "__flags__"}
+               "CHILL_TUNE_DQ_STREAMED", "CHILL_TUNE_DQ_STAGES", "CHILL_TUNE_DKDV_WAVES", "__flags__"}
     header = open(os.path.join(ROOT, "chill-attention_amd", "csrc", "chill_tiles.h")).read()
     for _, macros in tune.CANDIDATES:
         assert set(macros) <= allowed and all(m in header for m in macros if m != "__flags__")

@@ -457,22 +457,34 @@ DKDV_REGS_CASES = [
 ]
 
 
-@pytest.mark.parametrize("case", DKDV_REGS_CASES, ids=lambda c: c[0])
+# The same kernel at head dim 64 (rows of 128 bytes: one slab of a tile per wave, transposed operands of the two
+# 16-row halves at addresses of their own); chunkwise masks from chunks of 256 rows on
+DKDV_REGS_CASES_64 = [
+    ("causal", torch.bfloat16, 2, 16, 16, 4096, ("CausalChillMask", ()), None),
+    ("causal-gqa-lens-f16", torch.float16, 4, 16, 8, 4096, ("CausalChillMask", ()), (4096, 4000, 33, 2049)),
+    ("full-gqa-ragged", torch.bfloat16, 2, 32, 16, 4100, ("FullChillMask", ()), None),
+    ("prefix-lm-gqa-ragged-lens-f16", torch.float16, 1, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001,)),
+    ("long-prefix-lm", torch.bfloat16, 1, 32, 32, 8192, ("PrefixLMChillMask", (1024,)), None),
+    ("chunkwise-256x1-f16", torch.float16, 1, 32, 16, 8192, ("ChunkwiseChillMask", (256, 1)), (8000,)),
+]
+
+
+@pytest.mark.parametrize("case", [c + (128,) for c in DKDV_REGS_CASES] + [c + (64,) for c in DKDV_REGS_CASES_64],
+                         ids=lambda c: f"{c[0]}-D{c[-1]}")
 def test_dkdv_with_resident_keys_and_generated_loop(case):
     """The dK/dV kernel that keeps K in registers and runs its predicate-free tiles in a generated loop (and, from 8192
     keys on, the dQ kernel that does the same with Q and dO), on shapes the launcher routes to them (asserted from the
     tile table): heads of a GQA group one after the other, lens, sequence
     lengths that leave a ragged last tile, the first tiles of a key block under the mask (run by the ordinary code).
     Same bar as the other backward tests (chill_bwd_dkdv.py:347-508 is what it must equal)."""
-    _, dtype, B, H, Hkv, T, m, lens = case
-    D = 128
+    _, dtype, B, H, Hkv, T, m, lens, D = case
     mask = make_mask(m)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DKDV, seq_len=T, batch_heads=B * Hkv)
     assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
     # (dQ has such a kernel too, for sequences from 8192 on: the cases of that length below)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DQ, seq_len=T, batch_heads=B * H)
     banded = m[0] == "ChunkwiseChillMask"
-    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192 and not banded), f"dQ served by {cfg}"
+    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192 and not banded and D == 128), f"dQ served by {cfg}"
     torch.manual_seed(stable_seed(case[0]))
     q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
     lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)

@@ -95,6 +95,32 @@ def test_statement_declares_everything_it_writes(elem, D, waves, stages):
 
 
 @pytest.mark.parametrize("elem", ["bf16", "f16"])
+def test_backward_loop_at_head_dim_64(elem):
+    """The same generator at head dim 64: half the slots (32 MFMAs per iteration for the same vector work), one slab of a
+    tile per wave, and per-lane addresses of their own for the transposed operands of the two 16-row halves of a tile
+    (rows of 128 bytes: rows 16 apart do not share the swizzle key).  Every path passes the hazard check."""
+    c = genb.Config(elem, 64)
+    ins = genb.gen_statement(c)
+    outs, inputs, clob = genb.operand_lists(c)
+    genb.check_clobbers(ins, outs, clob + genb.SPECIAL_CLOBBERS, c.name)
+    names = [n for n, _ in inputs]
+    assert [n for n in names if n.startswith("qtr")] == [f"qtr{db}_{sx}_{w}" for db in range(2) for sx in range(2) for w in range(2)]
+    assert [n for n in names if n.startswith("g")] == ["gq0", "gdo0"] and sum(n.startswith("k") for n in names) == 8
+    cycle, orders = genb.find_steady_state(c)
+    it = genb.SteadyIteration(c, cycle[0], orders[-1])
+    st = genb.Stream()
+    it.generate(st, 0)
+    text = [i["text"] for i in st.ins]
+    assert sum(t.startswith("v_mfma") for t in text) == 32 and sum(t.startswith("v_exp_f32") for t in text) == 32
+    assert sum(t.startswith("ds_read_b128") for t in text) == 4 + 4 + 8 + 4 + 8 and sum(t.startswith("ds_read_b64_tr_b16") for t in text) == 16
+    assert sum(t.startswith("global_load_lds_dwordx4") for t in text) == 2
+    # no transposed read adds a half-tile offset to its address
+    tr = [t for t in text if t.startswith("ds_read_b64_tr_b16")]
+    assert all(int(t.split("offset:")[1]) % c.stage in (0, c.tile) for t in tr)
+    assert f"s_waitcnt vmcnt({c.loads_per_tile})" in text and c.loads_per_tile == 2
+
+
+@pytest.mark.parametrize("elem", ["bf16", "f16"])
 def test_backward_loop_generates_and_declares_what_it_writes(elem):
     """The generated loop of the dK/dV kernel with register-resident K (csrc/gen_bwd_loop.py): every path through the
     statement (prologue of each stage, its iteration, the next ones, the exit) passes the hazard check, the ring of
