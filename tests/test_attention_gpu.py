@@ -545,16 +545,17 @@ def test_gradients_through_strided_and_fp32_dout():
         torch.testing.assert_close(got, want.half(), atol=5e-3, rtol=1e-3)
 
 
-def test_register_resident_backward_on_strided_views():
-    """The long-sequence backward kernels at head dim 128 (K, or Q and dO, in registers; tile pointers that the generated
+@pytest.mark.parametrize("D", [128, 64])
+def test_register_resident_backward_on_strided_views(D):
+    """The long-sequence backward kernels (K, or at head dim 128 Q and dO, in registers; tile pointers that the generated
     loops move on by a row stride) on [B, T, H, D] storage viewed as [B, H, T, D], a GQA group, and an upstream gradient
     with a padded row pitch: bit for bit what the same launch gives on contiguous copies."""
     mask = ca.CausalChillMask()
-    B, H, Hkv, T, D = 2, 16, 8, 8192, 128
+    B, H, Hkv, T = 2, 16, 8, 8192
     dtype = torch.bfloat16
     for pss, cfg_heads in ((_lib.PASS_DKDV, B * Hkv), (_lib.PASS_DQ, B * H)):
         cfg = tile_config(mask, D, dtype, pss, seq_len=T, batch_heads=cfg_heads)
-        assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
+        assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (D == 128 or pss == _lib.PASS_DKDV), f"served by {cfg}"
     torch.manual_seed(11)
     q = torch.randn(B, T, H, D, device=DEV, dtype=dtype).transpose(1, 2).requires_grad_()
     k, v = (torch.randn(B, T, Hkv, D, device=DEV, dtype=dtype).transpose(1, 2).requires_grad_() for _ in range(2))
