@@ -282,22 +282,27 @@ constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
 // T4096 0.98 / 1.16, prefix-LM B4 H16 T8192 1.91 / 2.16; but causal B1 H8 T8192 0.368 / 0.318, B4 H16 T2048
 // 0.227 / 0.197, sliding window 512 at T8192 0.65 / 0.49.  At head dim 64 (against the 4-wave kernel that runs three
 // to a CU): causal B8 H16 T4096 0.73 / 0.77, B4 H32 T8192 2.12 / 2.42, B2 H8 T8192 0.31 / 0.36, B1 H32 T16384 1.99 / 2.35,
-// full mask B4 H16 T4096 0.56 / 0.73, prefix-LM B4 H32 T8192 2.12 / 2.45.
+// full mask B4 H16 T4096 0.56 / 0.73, prefix-LM B4 H32 T8192 2.12 / 2.45; there the other kernel's workgroups are a
+// quarter of the size and fill a small grid better: B2 H16 T4096 (512 workgroups of this kernel) causal 0.20 / 0.17,
+// prefix-LM 0.20 / 0.18 (but full mask 0.28 / 0.38); B4 H16 T4096 (1024) causal 0.37 / 0.38: from four workgroups per CU on.
 constexpr int kDkdvRegsBlocks128 = 2;
 constexpr int kDkdvRegsMinSequence = 4096;
 constexpr int kDkdvRegsMinWorkgroups = 2 * 256;
+constexpr int kDkdvRegsMinWorkgroups64 = 4 * 256;
 constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && (D == 128 || D == 64); }
 // Banded masks take it only when a wave's 64 key rows lie in one chunk, so that its tiles are all predicate-free
 // and all alike: chunkwise masks whose chunk size is a multiple of 64 (`mask_arg0` = the mask's first argument;
 // measured at head dim 128, T = 8192 and 16384: chunks of 64 / 128 / 256 / 1024 rows -5 / -8 / -13 / -16 %, chunks
 // of 96 rows +13 %, sliding windows of 64 .. 512 rows +32 .. +60 %, of 1024 rows and more +-1 %; at head dim 64,
-// where a tile is half the work, chunks of 64 rows +30 .. +68 %, of 128 rows +-1 %, of 1024 rows -17 %: from 256 rows on).
+// where a tile is half the work, chunks of 64 rows +30 .. +68 %, of 128 rows +-1 %, of 256 rows 0 .. +8 %, of 320 rows
+// -8 %, of 512 rows -19 %, of 1024 rows -17 %: from 320 rows on).
 constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0, int D) {
-    return mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0 && (D >= 128 || mask_arg0 >= 256);
+    return mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0 && (D >= 128 || mask_arg0 >= 320);
 }
 constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, int D, long long batch_kv_heads, int T) {
     return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, D)) && T >= kDkdvRegsMinSequence &&
-           batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >= kDkdvRegsMinWorkgroups;
+           batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >=
+               (D >= 128 ? kDkdvRegsMinWorkgroups : kDkdvRegsMinWorkgroups64);
 }
 
 // `regs`: the row of dkdv_regs_kernel where that kernel is an option (dkdv_regs_is_optional)

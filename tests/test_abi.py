@@ -176,14 +176,15 @@ def test_tile_table():
     assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, None) == -1
     desc.nargs = 1
     assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == -4
-    # the same kernel at head dim 64 (rows of 128 bytes), for the same launches; of the chunkwise masks only chunks of
-    # 256 rows and more
+    # the same kernel at head dim 64 (rows of 128 bytes), on grids of at least four workgroups per CU; of the chunkwise
+    # masks only chunks of 320 rows and more
     regs64 = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 256 * 128 + 4 * (2 * 32 * 128 + 2 * 32 * 4)}
     assert tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV) == regs64
     assert tile_config(ca.PrefixLMChillMask(1024), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
-    assert tile_config(ca.ChunkwiseChillMask(256, 1), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
-    for mask, T, bh in ((causal, 4096, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64), (ca.ChunkwiseChillMask(64, 4), 8192, 64),
-                        (window, 8192, 128)):
+    assert tile_config(ca.ChunkwiseChillMask(512, 1), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
+    assert tile_config(causal, 64, torch.float16, _lib.PASS_DKDV, seq_len=4096, batch_heads=64) == regs64
+    for mask, T, bh in ((causal, 4096, 63), (causal, 8192, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64),
+                        (ca.ChunkwiseChillMask(256, 1), 8192, 128), (window, 8192, 128)):
         c = tile_config(mask, 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
         assert (c["rows"], c["waves"], c["streamed"]) == (64, 4, 64), (mask, T, bh, c)
     assert 2 * tile_config(window, 64, torch.bfloat16, _lib.PASS_DKDV)["lds_bytes"] <= 160 * 1024

@@ -458,14 +458,14 @@ DKDV_REGS_CASES = [
 
 
 # The same kernel at head dim 64 (rows of 128 bytes: one slab of a tile per wave, transposed operands of the two
-# 16-row halves at addresses of their own); chunkwise masks from chunks of 256 rows on
+# 16-row halves at addresses of their own), on grids of at least 1024 workgroups; chunkwise masks from chunks of 320 rows on
 DKDV_REGS_CASES_64 = [
-    ("causal", torch.bfloat16, 2, 16, 16, 4096, ("CausalChillMask", ()), None),
-    ("causal-gqa-lens-f16", torch.float16, 4, 16, 8, 4096, ("CausalChillMask", ()), (4096, 4000, 33, 2049)),
-    ("full-gqa-ragged", torch.bfloat16, 2, 32, 16, 4100, ("FullChillMask", ()), None),
-    ("prefix-lm-gqa-ragged-lens-f16", torch.float16, 1, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001,)),
+    ("causal", torch.bfloat16, 4, 16, 16, 4096, ("CausalChillMask", ()), None),
+    ("causal-gqa-lens-f16", torch.float16, 8, 16, 8, 4096, ("CausalChillMask", ()), (4096, 4000, 33, 2049, 4096, 1, 3111, 4095)),
+    ("full-gqa-ragged", torch.bfloat16, 4, 32, 16, 4100, ("FullChillMask", ()), None),
+    ("prefix-lm-gqa-ragged-lens-f16", torch.float16, 2, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001, 4111)),
     ("long-prefix-lm", torch.bfloat16, 1, 32, 32, 8192, ("PrefixLMChillMask", (1024,)), None),
-    ("chunkwise-256x1-f16", torch.float16, 1, 32, 16, 8192, ("ChunkwiseChillMask", (256, 1)), (8000,)),
+    ("chunkwise-512x1-f16", torch.float16, 2, 32, 16, 8192, ("ChunkwiseChillMask", (512, 1)), (8000, 8192)),
 ]
 
 
@@ -551,7 +551,7 @@ def test_register_resident_backward_on_strided_views(D):
     loops move on by a row stride) on [B, T, H, D] storage viewed as [B, H, T, D], a GQA group, and an upstream gradient
     with a padded row pitch: bit for bit what the same launch gives on contiguous copies."""
     mask = ca.CausalChillMask()
-    B, H, Hkv, T = 2, 16, 8, 8192
+    B, H, Hkv, T = (2, 16, 8, 8192) if D == 128 else (2, 32, 16, 8192)  # (head dim 64: on grids of 1024 workgroups)
     dtype = torch.bfloat16
     for pss, cfg_heads in ((_lib.PASS_DKDV, B * Hkv), (_lib.PASS_DQ, B * H)):
         cfg = tile_config(mask, D, dtype, pss, seq_len=T, batch_heads=cfg_heads)
