@@ -155,7 +155,8 @@ __global__ __launch_bounds__(256) void dkdv_regs_kernel(BwdParams p, int n_k_til
         load_resident<E, D>(kf[c], kptr + (int64_t)(kw + 32 * c) * p.sk.t, p.sk.t, p.T - kw - 32 * c, lane);
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
-    if (kw < seq_len) wr = tile_range<MASK, false>(kw, KPW, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
+    // (key rows of the wave at and beyond seq_len are computed like the others and stored as zeros)
+    if (kw < seq_len) wr = tile_range_rows_discarded<MASK, false>(kw, KPW, TQS, seq_len, wave_has_full_blocks != 0, p.margs);
     const int ta = wr.start - wg.start, tb = wr.end - wg.start;
     const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
 

@@ -166,7 +166,8 @@ __global__ __launch_bounds__(256) void dq_regs2_kernel(BwdParams p, int n_q_tile
     });
 
     TileRange wr = {wg.start, wg.start, wg.start, wg.start};
-    if (qw < seq_len) wr = tile_range<MASK, true>(qw, 32 * CB, TK, seq_len, wave_has_full_blocks != 0, p.margs);
+    // (rows of the wave at and beyond seq_len are computed like the others and never stored)
+    if (qw < seq_len) wr = tile_range_rows_discarded<MASK, true>(qw, 32 * CB, TK, seq_len, wave_has_full_blocks != 0, p.margs);
     const int ta = wr.start - wg.start, tb = wr.end - wg.start;
     const int fa = wr.full_start - wg.start, fb = wr.full_end - wg.start;
 

@@ -303,6 +303,32 @@ CHILL_HD TileRange tile_range(int i, int tile_in, int tile_out, int seq_len, boo
     return r;
 }
 
+// The same for a kernel that computes the rows of a ragged last row tile like any others and throws them
+// away: the rows of [i, i + tile_in) at and beyond seq_len exist in memory or read as zero, they are never
+// stored, and no row's result depends on another row's.  The predicate-free range of the COMPLETE tile
+// (every mask states it from the tile's first row and size) holds for the rows that exist, so the tile
+// need not end inside the sequence as the reference's loop split asks (chill_bwd_dq.py:279-293,
+// chill_bwd_dkdv.py:329-344); the streamed tiles of the range do lie inside it.  Without this the one
+// ragged workgroup of a head runs every tile under the predicate and finishes long after the others
+// (causal B4 H16 D128 dQ: T = 8192 1.39 ms, T = 8200 1.63 ms).
+template <int ID, bool QROWS>
+CHILL_HD TileRange tile_range_rows_discarded(int i, int tile_in, int tile_out, int seq_len, bool has_full_blocks,
+                                             MaskArgs a) {
+    using M = Mask<ID>;
+    TileRange r = tile_range<ID, QROWS>(i, tile_in, tile_out, seq_len, has_full_blocks, a);
+    constexpr bool kSplit = QROWS ? M::kHasKFullRange : M::kHasQFullRange;
+    if (kSplit && has_full_blocks && i + tile_in > seq_len) {
+        const Range f = QROWS ? M::k_full_range_for_q(i, tile_in, seq_len, a) : M::q_full_range_for_k(i, tile_in, seq_len, a);
+        const int fs = imax(r.start, cdiv(f.lo, tile_out));
+        const int fe = imin(imin(r.end, f.hi / tile_out), seq_len / tile_out);
+        if (fs < fe) {
+            r.full_start = fs;
+            r.full_end = fe;
+        }
+    }
+    return r;
+}
+
 // has_full_blocks for a pass: the row tile is (tq) for QROWS passes and (tk) for the dK/dV pass,
 // but the mask rule always takes (q_tile, k_tile) in that order (chill.py:159-164, 375-386).
 template <int ID>
