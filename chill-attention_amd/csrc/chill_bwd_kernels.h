@@ -1398,7 +1398,8 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
         constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DKDV);
         if constexpr (served) small = bwd_takes_small((long long)p.B * p.H_kv, p.T, D, Elem<E>::kDType, CHILL_PASS_DKDV);
         bool regs = false;
-        if constexpr (dkdv_regs_is_optional(D, Elem<E>::kDType)) regs = dkdv_takes_regs(MASK_ID, p.margs.a0, D, (long long)p.B * p.H_kv, p.T);
+        if constexpr (dkdv_regs_is_optional(D, Elem<E>::kDType))
+            regs = dkdv_takes_regs(MASK_ID, p.margs.a0, mask_band_keys(MASK_ID, p.margs.a0, p.margs.a1), D, (long long)p.B * p.H_kv, p.T);
         if (small) {
             if constexpr (served) status = launch_bwd_small<E, D, MASK_ID, 2>(p, stream);
         } else if (regs) {

@@ -527,8 +527,9 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         if (small) {
             if constexpr (D * Elem<E>::kBytes <= 512) status = launch_fwd_small<E, D, MASK_ID>(p, stream);
         } else if constexpr (has_short_row) {
-            status = fwd_takes_short_row((long long)p.B * p.H, p.T) ? launch_fwd_shape<E, D, MASK_ID, true>(p, stream)
-                                                                    : launch_fwd_shape<E, D, MASK_ID, false>(p, stream);
+            const bool short_row = fwd_takes_short_row(MASK_ID, mask_band_keys(MASK_ID, p.margs.a0, p.margs.a1),
+                                                       (long long)p.B * p.H, p.T);
+            status = short_row ? launch_fwd_shape<E, D, MASK_ID, true>(p, stream) : launch_fwd_shape<E, D, MASK_ID, false>(p, stream);
         } else {
             status = launch_fwd_shape<E, D, MASK_ID, false>(p, stream);
         }

@@ -121,13 +121,13 @@ int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, i
     return chill_tile_config_for_shape(mask_id, D, dtype, pass, 1, kLongSequence, out);
 }
 
-static int report_tile_config(int mask_id, long long mask_arg0, int32_t D, int32_t dtype, int32_t pass,
+static int report_tile_config(int mask_id, long long mask_arg0, long long band_keys, int32_t D, int32_t dtype, int32_t pass,
                               int64_t batch_heads, int32_t T, int32_t out[4]) {
     if (out == nullptr) return CHILL_ERR_NULL_POINTER;
     if (!mask_id_served(mask_id)) return CHILL_ERR_BAD_MASK;
     if (T < 1 || batch_heads < 1) return CHILL_ERR_BAD_ARGUMENT;
     TileConfig c;
-    int st = tile_config(mask_id, mask_arg0, D, dtype, pass, batch_heads, T, &c);
+    int st = tile_config(mask_id, mask_arg0, band_keys, D, dtype, pass, batch_heads, T, &c);
     if (st != CHILL_OK) return st;
     out[0] = c.rows;
     out[1] = c.streamed;
@@ -138,8 +138,8 @@ static int report_tile_config(int mask_id, long long mask_arg0, int32_t D, int32
 
 int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
                                 int32_t T, int32_t out[4]) {
-    // (a mask id alone: the row of a mask whose arguments do not change the route)
-    return report_tile_config(mask_id, 1, D, dtype, pass, batch_heads, T, out);
+    // (a mask id alone: the row of a mask whose arguments do not change the route; of a banded mask, a narrow one)
+    return report_tile_config(mask_id, 1, mask_is_banded(mask_id) ? kNarrowBand : kWholeSequence, D, dtype, pass, batch_heads, T, out);
 }
 
 int chill_tile_config_for_launch(const ChillMaskDesc* mask, int32_t D, int32_t dtype, int32_t pass,
@@ -147,7 +147,7 @@ int chill_tile_config_for_launch(const ChillMaskDesc* mask, int32_t D, int32_t d
     MaskArgs a;
     int st = lower_mask(mask, &a);
     if (st != CHILL_OK) return st;
-    return report_tile_config(mask->id, a.a0, D, dtype, pass, batch_heads, T, out);
+    return report_tile_config(mask->id, a.a0, mask_band_keys(mask->id, a.a0, a.a1), D, dtype, pass, batch_heads, T, out);
 }
 
 const char* chill_status_string(int32_t status) {

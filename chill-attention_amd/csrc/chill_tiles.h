@@ -65,6 +65,16 @@ constexpr int fwd_stage_bytes(int streamed, int D, int dtype) {
 constexpr bool mask_is_banded(int mask_id) {
     return mask_id == CHILL_MASK_SLIDING_WINDOW || mask_id == CHILL_MASK_CHUNKWISE;
 }
+// The most keys a row of such a mask sees (`a0`, `a1` = the mask's first two arguments: left and right context, or
+// chunk size and chunks looked back at); kWholeSequence for the other masks.  A wide band is a long loop again:
+// the forward and dK/dV then take the shapes of the masks that are not banded, from the widths named at
+// fwd_takes_short_row and dkdv_regs_serves_band on.
+constexpr long long kWholeSequence = 1ll << 40;
+constexpr long long mask_band_keys(int mask_id, long long a0, long long a1) {
+    return mask_id == CHILL_MASK_SLIDING_WINDOW ? a0 + a1 + 1 : mask_id == CHILL_MASK_CHUNKWISE ? a0 * (a1 + 1) : kWholeSequence;
+}
+// (a banded mask of which only the id is known is taken to be narrow)
+constexpr long long kNarrowBand = 1;
 
 // Sequence lengths up to which the 4-wave shape also wins at head dim 128 for masks that are not banded
 // (measured on causal and full masks, B8 H4 .. H16: forward -16 % at T = 512 and 1024, +20 % at 2085;
@@ -78,22 +88,27 @@ constexpr int kDqShortSequence = 4096;
 constexpr int kComputeUnits = 256;
 // (forward: only dQ still takes it; the 8-wave forward with its generated loop is 23 % faster than the 4-wave
 // one at B1 H8 T8192)
-constexpr bool fwd_takes_short_row(long long batch_heads, int T) {
+// Banded masks take it while a row sees fewer than kFwdWideBand keys (measured at head dim 128, T = 8192 and 16384,
+// the 8-wave shape against this one: sliding windows of 512 / 1024 / 2048 / 4096 keys +9 / -12 / -18 / -18 %,
+// chunkwise 1024 x 2 -17 %, 128 x 3 +2 %).
+constexpr int kFwdWideBand = 1024;
+constexpr bool fwd_takes_short_row(int mask_id, long long band_keys, long long batch_heads, int T) {
     (void)batch_heads;
-    return T <= kFwdShortSequence;
+    return T <= kFwdShortSequence || (mask_is_banded(mask_id) && band_keys < kFwdWideBand);
 }
 constexpr bool dq_takes_short_row(long long batch_heads, int T) {
     return T <= kDqShortSequence || batch_heads * ((T + 255) / 256) <= kComputeUnits;
 }
 
 // Forward.  16-bit inputs at head dim 128: 8 waves (256 query rows), streamed tiles of 128 keys (half
-// the barriers per key); banded masks, head dims <= 64 and short sequences: 4 waves, 64 keys, 2
+// the barriers per key); narrow bands (fwd_takes_short_row), head dims <= 64 and short sequences: 4 waves, 64 keys, 2
 // stages, two or three workgroups per CU (prefix-LM at D = 64: forward -14 %; causal at D = 16 .. 64:
 // -5 .. -8 %).
 constexpr int fwd_waves(int mask_id, int D, int dtype, int T) {
     if (dtype == CHILL_F32 || D > 128) return 4;
     if (CHILL_TUNE_FWD_WAVES) return CHILL_TUNE_FWD_WAVES;
-    return (mask_is_banded(mask_id) || D <= 64 || T <= kFwdShortSequence) ? 4 : 8;
+    (void)mask_id;
+    return (D <= 64 || T <= kFwdShortSequence) ? 4 : 8;
 }
 constexpr int fwd_streamed(int mask_id, int D, int dtype, int T) {
     if (dtype == CHILL_F32) return 32;
@@ -293,14 +308,17 @@ constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F
 // Banded masks take it only when a wave's 64 key rows lie in one chunk, so that its tiles are all predicate-free
 // and all alike: chunkwise masks whose chunk size is a multiple of 64 (`mask_arg0` = the mask's first argument;
 // measured at head dim 128, T = 8192 and 16384: chunks of 64 / 128 / 256 / 1024 rows -5 / -8 / -13 / -16 %, chunks
-// of 96 rows +13 %, sliding windows of 64 .. 512 rows +32 .. +60 %, of 1024 rows and more +-1 %; at head dim 64,
-// where a tile is half the work, chunks of 64 rows +30 .. +68 %, of 128 rows +-1 %, of 256 rows 0 .. +8 %, of 320 rows
-// -8 %, of 512 rows -19 %, of 1024 rows -17 %: from 320 rows on).
-constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0, int D) {
-    return mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0 && (D >= 128 || mask_arg0 >= 320);
+// of 96 rows +13 %; at head dim 64, where a tile is half the work, chunks of 64 rows +30 .. +68 %, of 128 rows +-1 %,
+// of 256 rows 0 .. +8 %, of 320 rows -8 %, of 512 rows -19 %, of 1024 rows -17 %: from 320 rows on); and sliding
+// windows from kDkdvRegsWideBand keys on (`band_keys` = mask_band_keys; windows of 64 .. 512 keys +32 .. +60 %,
+// of 1024 +14 %, of 2048 -2 %, of 4096 -8 % at head dim 128 and -11 % at head dim 64).
+constexpr int kDkdvRegsWideBand = 4096;
+constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0, long long band_keys, int D) {
+    return (mask_id == CHILL_MASK_CHUNKWISE && mask_arg0 % (32 * kDkdvRegsBlocks128) == 0 && (D >= 128 || mask_arg0 >= 320)) ||
+           (mask_id == CHILL_MASK_SLIDING_WINDOW && band_keys >= kDkdvRegsWideBand);
 }
-constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, int D, long long batch_kv_heads, int T) {
-    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, D)) && T >= kDkdvRegsMinSequence &&
+constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, long long band_keys, int D, long long batch_kv_heads, int T) {
+    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, band_keys, D)) && T >= kDkdvRegsMinSequence &&
            batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >=
                (D >= 128 ? kDkdvRegsMinWorkgroups : kDkdvRegsMinWorkgroups64);
 }
@@ -325,9 +343,10 @@ constexpr TileConfig dkdv_tile_config(int mask_id, int D, int dtype, bool small_
 
 // batch_heads = B * H and T = sequence length of the launch (the forward and dQ rows depend on them);
 // T = kLongSequence for the row of long sequences on a full chip.
-// mask_arg0 = the mask's first argument (the dK/dV row of chunkwise masks depends on the chunk size).
-inline int tile_config(int mask_id, long long mask_arg0, int D, int dtype, int pass, long long batch_heads, int T,
-                       TileConfig* out) {
+// mask_arg0 = the mask's first argument (the dK/dV row of chunkwise masks depends on the chunk size), band_keys =
+// mask_band_keys of the mask (the forward and dK/dV rows of banded masks depend on the width of the band).
+inline int tile_config(int mask_id, long long mask_arg0, long long band_keys, int D, int dtype, int pass, long long batch_heads,
+                       int T, TileConfig* out) {
     if (dtype != CHILL_F32 && dtype != CHILL_F16 && dtype != CHILL_BF16) return CHILL_ERR_BAD_DTYPE;
     if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
     switch (pass) {
@@ -336,7 +355,7 @@ inline int tile_config(int mask_id, long long mask_arg0, int D, int dtype, int p
                 *out = TileConfig{32, 32, kFwdSmallWaves, fwd_small_lds_bytes(D, dtype)};
                 return CHILL_OK;
             }
-            *out = fwd_tile_config(mask_id, D, dtype, (T != kLongSequence && fwd_takes_short_row(batch_heads, T)) ? 1 : kLongSequence);
+            *out = fwd_tile_config(mask_id, D, dtype, fwd_takes_short_row(mask_id, band_keys, batch_heads, T) ? 1 : kLongSequence);
             return CHILL_OK;
         case CHILL_PASS_DQ:
             if (T != kLongSequence && bwd_takes_small(batch_heads, T, D, dtype, CHILL_PASS_DQ)) {
@@ -357,8 +376,8 @@ inline int tile_config(int mask_id, long long mask_arg0, int D, int dtype, int p
             }
             // (the row of long sequences on a full chip: the generated loop where there is one)
             *out = dkdv_tile_config(mask_id, D, dtype, T != kLongSequence && dkdv_takes_small_row(batch_heads, T),
-                                    T == kLongSequence ? (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, D))
-                                                       : dkdv_takes_regs(mask_id, mask_arg0, D, batch_heads, T));
+                                    T == kLongSequence ? (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, band_keys, D))
+                                                       : dkdv_takes_regs(mask_id, mask_arg0, band_keys, D, batch_heads, T));
             return CHILL_OK;
         default: return CHILL_ERR_BAD_ARGUMENT;
     }

@@ -231,7 +231,10 @@ int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32
 /* The same for one launch with its mask: the dK/dV row of a chunkwise mask depends on the chunk size (with
  * chunks of a multiple of 64 rows a wave's key rows lie in one chunk, no block inside its band is partly
  * masked, and the launch takes the kernel with the generated loop at head dim 128;
- * chill_tile_config_for_shape reports the row of the other chunk sizes).
+ * chill_tile_config_for_shape reports the row of the other chunk sizes), and the forward and dK/dV rows of
+ * a banded mask on the most keys a row sees (from 1024 keys on the forward at head dim 128 takes the row of
+ * the masks that are not banded, from 4096 keys on so does dK/dV under a sliding window;
+ * chill_tile_config_for_shape reports the rows of a narrow band).
  * Counterpart of the autotuner's key, which includes the mask's constants (autotune.py:129-240). */
 int chill_tile_config_for_launch(const ChillMaskDesc* mask, int32_t D, int32_t dtype, int32_t pass,
                                  int64_t batch_heads, int32_t T, int32_t out[4]);

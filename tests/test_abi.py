@@ -167,8 +167,23 @@ def test_tile_table():
                         (ca.ChunkwiseChillMask(128, 2), 4096, 31), (ca.ChunkwiseChillMask(128, 2), None, 1 << 20)):
         c = tile_config(mask, 128, torch.float16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
         assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
+    # a banded mask whose rows see many keys is a long loop again: the forward at head dim 128 takes its 8-wave shape from
+    # 1024 keys on, dK/dV under a sliding window its register-resident kernel from 4096 keys on (dQ keeps the 4-wave shape)
+    for mask, waves in ((ca.SlidingWindowChillMask(1023, 0), 8), (ca.SlidingWindowChillMask(1000, 22), 4), (ca.SlidingWindowChillMask(128, 128), 4),
+                        (ca.ChunkwiseChillMask(512, 1), 8), (ca.ChunkwiseChillMask(128, 2), 4), (ca.ChunkwiseChillMask(341, 2), 4)):
+        assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_FWD, seq_len=8192, batch_heads=128)["waves"] == waves, mask
+        assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_FWD, seq_len=1024, batch_heads=128)["waves"] == 4, mask
+        assert tile_config(mask, 64, torch.bfloat16, _lib.PASS_FWD, seq_len=8192, batch_heads=128)["waves"] == 4, mask
+        assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_DQ, seq_len=8192, batch_heads=128)["waves"] == 4, mask
+    assert tile_config(ca.SlidingWindowChillMask(4095, 0), 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs
+    assert tile_config(ca.SlidingWindowChillMask(2000, 2095), 128, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs
+    for mask, T, bh in ((ca.SlidingWindowChillMask(4094, 0), 8192, 128), (ca.SlidingWindowChillMask(4095, 0), 4095, 128),
+                        (ca.SlidingWindowChillMask(4095, 0), 8192, 15)):
+        c = tile_config(mask, 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
+        assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
     out4 = (ctypes.c_int32 * 4)()
     assert _lib.lib.chill_tile_config_for_shape(3, 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == 0 and out4[0] == 128
+    assert _lib.lib.chill_tile_config_for_shape(2, 128, _lib.F16, _lib.PASS_FWD, 64, 16384, out4) == 0 and out4[2] == 4
     desc = ca.ChunkwiseChillMask(128, 2).descriptor()
     assert _lib.lib.chill_tile_config_for_launch(ctypes.byref(desc), 128, _lib.F16, _lib.PASS_DKDV, 64, 16384, out4) == 0
     assert list(out4) == [regs["rows"], regs["streamed"], regs["waves"], regs["lds_bytes"]]
@@ -183,6 +198,7 @@ def test_tile_table():
     assert tile_config(ca.PrefixLMChillMask(1024), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     assert tile_config(ca.ChunkwiseChillMask(512, 1), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     assert tile_config(causal, 64, torch.float16, _lib.PASS_DKDV, seq_len=4096, batch_heads=64) == regs64
+    assert tile_config(ca.SlidingWindowChillMask(4096, 100), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     for mask, T, bh in ((causal, 4096, 63), (causal, 8192, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64),
                         (ca.ChunkwiseChillMask(256, 1), 8192, 128), (window, 8192, 128)):
         c = tile_config(mask, 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)

@@ -454,6 +454,9 @@ DKDV_REGS_CASES = [
     ("chunkwise-64x4-gqa-lens", torch.bfloat16, 4, 16, 8, 4096, ("ChunkwiseChillMask", (64, 4)), (4096, 3000, 77, 4001)),
     ("chunkwise-1024x1-ragged-f16", torch.float16, 1, 32, 32, 4140, ("ChunkwiseChillMask", (1024, 1)), None),
     ("chunkwise-192x0", torch.bfloat16, 1, 32, 32, 4096, ("ChunkwiseChillMask", (192, 0)), None),
+    # sliding windows of 4096 keys and more: a long loop again, with masked tiles at both ends of a wave's run
+    ("sliding-4096+0", torch.bfloat16, 2, 16, 16, 8192, ("SlidingWindowChillMask", (4096, 0)), None),
+    ("sliding-3000+2000-gqa-ragged-lens-f16", torch.float16, 1, 32, 16, 8200, ("SlidingWindowChillMask", (3000, 2000)), (8100,)),
 ]
 
 
@@ -466,7 +469,48 @@ DKDV_REGS_CASES_64 = [
     ("prefix-lm-gqa-ragged-lens-f16", torch.float16, 2, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001, 4111)),
     ("long-prefix-lm", torch.bfloat16, 1, 32, 32, 8192, ("PrefixLMChillMask", (1024,)), None),
     ("chunkwise-512x1-f16", torch.float16, 2, 32, 16, 8192, ("ChunkwiseChillMask", (512, 1)), (8000, 8192)),
+    ("sliding-4096+100", torch.bfloat16, 2, 32, 32, 8192, ("SlidingWindowChillMask", (4096, 100)), None),
 ]
+
+
+# Banded masks whose rows see 1024 keys and more take the forward's 8-wave shape with its generated loop at head dim 128
+# (narrower ones keep the 4-wave shape): runs of predicate-free tiles with masked tiles before and after them, waves of one
+# workgroup whose runs differ, chunk sizes that are no multiple of a tile, a band wider than the sequence
+WIDE_BAND_FWD_CASES = [
+    ("sliding-1024+0", torch.bfloat16, 2, 4, 4, 4096, ("SlidingWindowChillMask", (1024, 0)), None, (256, 8)),
+    ("sliding-700+700-ragged-lens-f16", torch.float16, 2, 4, 2, 4133, ("SlidingWindowChillMask", (700, 700)), (4133, 2500), (256, 8)),
+    ("sliding-5000+0-wider-than-T", torch.bfloat16, 1, 8, 8, 3000, ("SlidingWindowChillMask", (5000, 0)), None, (256, 8)),
+    ("chunkwise-1000x1-f16", torch.float16, 1, 8, 8, 4096, ("ChunkwiseChillMask", (1000, 1)), None, (256, 8)),
+    ("chunkwise-512x1-gqa-lens", torch.bfloat16, 2, 8, 2, 4096, ("ChunkwiseChillMask", (512, 1)), (4000, 1111), (256, 8)),
+    ("sliding-1000+22-narrow", torch.bfloat16, 1, 8, 8, 4096, ("SlidingWindowChillMask", (1000, 22)), None, (128, 4)),
+    ("chunkwise-256x2-narrow-f16", torch.float16, 1, 8, 8, 4096, ("ChunkwiseChillMask", (256, 2)), None, (128, 4)),
+]
+
+
+@pytest.mark.parametrize("case", WIDE_BAND_FWD_CASES, ids=lambda c: c[0])
+def test_forward_of_wide_bands_takes_the_long_loop(case):
+    """O and LSE2 (chill_fwd.py:215-330 is what they must equal) and the gradients behind them on banded masks either
+    side of the width from which the forward takes the shape of the masks that are not banded (route asserted)."""
+    _, dtype, B, H, Hkv, T, m, lens, route = case
+    D = 128
+    mask = make_mask(m)
+    cfg = tile_config(mask, D, dtype, _lib.PASS_FWD, seq_len=T, batch_heads=B * H)
+    assert (cfg["rows"], cfg["waves"]) == route, f"served by {cfg}"
+    torch.manual_seed(stable_seed(case[0]))
+    q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    dout = torch.randn(B, H, T, D, device=DEV, dtype=dtype)
+    out, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens_t, return_lse=True)
+    out.backward(dout)
+    qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+    ref, res_mask = orc.reference_naive(m[0], m[1], qf, kf, vf, lens_t)
+    ref.backward(dout.float() * res_mask)
+    check_close(out.detach() * res_mask, ref.detach(), dtype, OUT_TOL[dtype], D, "O")
+    want_lse = orc.lse2_dense(m[0], m[1], q.detach(), k.detach(), lens_t)
+    seen = torch.isfinite(want_lse)  # (rows at and behind lens see no key)
+    torch.testing.assert_close(lse[seen].double(), want_lse[seen], atol=2e-2, rtol=1e-3)
+    for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
+        check_close(got, want, dtype, GRAD_TOL[dtype], D, name)
 
 
 @pytest.mark.parametrize("case", [c + (128,) for c in DKDV_REGS_CASES] + [c + (64,) for c in DKDV_REGS_CASES_64],
@@ -483,7 +527,7 @@ def test_dkdv_with_resident_keys_and_generated_loop(case):
     assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
     # (dQ has such a kernel too, for sequences from 8192 on: the cases of that length below)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DQ, seq_len=T, batch_heads=B * H)
-    banded = m[0] == "ChunkwiseChillMask"
+    banded = m[0] in ("ChunkwiseChillMask", "SlidingWindowChillMask")
     assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192 and not banded and D == 128), f"dQ served by {cfg}"
     torch.manual_seed(stable_seed(case[0]))
     q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
