@@ -513,6 +513,66 @@ def test_forward_of_wide_bands_takes_the_long_loop(case):
         check_close(got, want, dtype, GRAD_TOL[dtype], D, name)
 
 
+def _random_long_cases(n, seed):
+    """Seeded draws of (head dim, dtype, B, H, H_kv, T, mask, lens) among the shapes the launchers send to the kernels of long
+    sequences: most grids above the thresholds of the register-resident kernels, some below; ragged lengths; every mask
+    family with arguments either side of the widths and chunk sizes that change the route."""
+    import random
+
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n):
+        D = rng.choice([64, 128, 128])
+        dtype = rng.choice([torch.bfloat16, torch.float16])
+        T = rng.choice([4096, 4100, 5000, 6143, 8192, 8200, 9000, rng.randint(4096, 9500)])
+        m = rng.choice([
+            ("CausalChillMask", ()), ("FullChillMask", ()),
+            ("PrefixLMChillMask", (rng.choice([1, 77, 1024, 3000, 5000]),)),
+            ("SlidingWindowChillMask", (rng.choice([1023, 2048, 4096, 5000]), rng.choice([0, 0, 100, 2000]))),
+            ("SlidingWindowChillMask", (rng.choice([0, 64, 500]), rng.choice([0, 64, 300]))),
+            ("ChunkwiseChillMask", (rng.choice([64, 128, 320, 512, 1024]), rng.choice([0, 1, 3]))),
+            ("ChunkwiseChillMask", (rng.choice([96, 100, 333, 1000]), rng.choice([0, 2]))),
+            ("ChunkwiseChillMask", (rng.choice([512, 2048]), rng.choice([1, 2])))])
+        group = rng.choice([1, 1, 2, 4])
+        need = (512 if D == 128 else 1024) * 256 // T + 1  # B * H_kv from which dK/dV takes its register-resident kernel
+        if rng.random() < 0.25:
+            need = max(1, need // 4)
+        B = rng.choice([1, 2, 4])
+        Hkv = max(1, -(-need // B))
+        H = Hkv * group
+        if B * H * T * D * 2 > 400e6:
+            H = max(group, int(400e6 / (B * T * D * 2)) // group * group)
+            Hkv = H // group
+        lens = None
+        if rng.random() < 0.4:
+            lens = tuple(rng.choice([T, T - 1, rng.randint(1, T), rng.randint(T // 2, T)]) for _ in range(B))
+        cases.append((f"{i}-D{D}-{str(dtype)[6:]}-B{B}-H{H}/{Hkv}-T{T}-{m[0][:-9]}{list(m[1])}", D, dtype, B, H, Hkv, T, m, lens))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_long_cases(32, 20240607), ids=lambda c: c[0])
+def test_random_long_sequences(case):
+    """Forward and backward against the dense reference (chill_fwd.py:215-330, chill_bwd_dq.py:300-394,
+    chill_bwd_dkdv.py:347-508 are what they must equal) on seeded random draws of long shapes."""
+    _, D, dtype, B, H, Hkv, T, m, lens = case
+    mask = make_mask(m)
+    torch.manual_seed(stable_seed(case[0]))
+    q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    dout = torch.randn(B, H, T, D, device=DEV, dtype=dtype)
+    out = ca.chill_attention(q, k, v, mask=mask, lens=lens_t)
+    out.backward(dout)
+    qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+    ref, res_mask = orc.reference_naive(m[0], m[1], qf, kf, vf, lens_t)
+    ref.backward(dout.float() * res_mask)
+    check_close(out.detach() * res_mask, ref.detach(), dtype, OUT_TOL[dtype], D, "O")
+    for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
+        check_close(got, want, dtype, GRAD_TOL[dtype], D, name)
+    if lens is not None:
+        for b, n in enumerate(lens):
+            assert (k.grad[b, :, n:] == 0).all() and (v.grad[b, :, n:] == 0).all() and (q.grad[b, :, n:] == 0).all()
+
+
 @pytest.mark.parametrize("case", [c + (128,) for c in DKDV_REGS_CASES] + [c + (64,) for c in DKDV_REGS_CASES_64],
                          ids=lambda c: f"{c[0]}-D{c[-1]}")
 def test_dkdv_with_resident_keys_and_generated_loop(case):
