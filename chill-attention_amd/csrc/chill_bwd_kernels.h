@@ -419,21 +419,32 @@ int launch_dq_regs2(const BwdParams& p, hipStream_t stream) {
 // PASS 1: dQ (workgroups over query blocks), 2: dK/dV (over key blocks).
 template <typename E, int D, int MASK_ID, int PASS>
 int launch_bwd_small(const BwdParams& p, hipStream_t stream) {
-    constexpr int kLdsBytes = bwd_small_lds_bytes(D, Elem<E>::kDType, PASS);
+    constexpr int kLdsOne = bwd_small_lds_bytes(D, Elem<E>::kDType, PASS);
     const int n_tiles = cdiv(p.T, 32);
-    const int total = p.B * (PASS == 1 ? p.H : p.H_kv) * n_tiles;  // (small by bwd_takes_small)
+    const long long heads = (long long)p.B * (PASS == 1 ? p.H : p.H_kv);  // (few by bwd_takes_small)
+    // (dK/dV keeps one block per workgroup: with K, V and two accumulators a wave needs more than the 256 registers it
+    // would be left with)
+    constexpr bool kTwoFit = PASS == 1 && small_fits_two_tiles(kLdsOne);
+    bool two = false;
+    if constexpr (kTwoFit) two = small_takes_two_tiles(heads * n_tiles);
+    const int total = (int)(heads * (two ? (n_tiles + 1) / 2 : n_tiles));
+    const int lds_bytes = two ? 2 * kLdsOne : kLdsOne;
     void (*kern)(BwdParams, int, int, int);
     if constexpr (PASS == 1)
-        kern = dq_small_kernel<E, D, MASK_ID>;
+        kern = dq_small_kernel<E, D, MASK_ID, 1>;
     else
         kern = dkdv_small_kernel<E, D, MASK_ID>;
+    if constexpr (kTwoFit) {
+        if (two) kern = dq_small_kernel<E, D, MASK_ID, 2>;
+    }
     const bool hfb = Mask<MASK_ID>::has_full_blocks(32, 32, p.T, p.margs);
-    if (kLdsBytes > 48 * 1024) {
+    if (lds_bytes > 48 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kLdsBytes) != hipSuccess)
+                                lds_bytes) != hipSuccess)
             return CHILL_ERR_HIP;
     }
-    hipLaunchKernelGGL(kern, dim3(total), dim3(kFwdSmallWaves * 64), kLdsBytes, stream, p, n_tiles, total, hfb ? 1 : 0);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(kFwdSmallWaves * 64 * (two ? 2 : 1)), lds_bytes, stream, p, n_tiles, total,
+                       hfb ? 1 : 0);
     return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
 }
 
@@ -448,7 +459,7 @@ int launch_dq(const BwdParams& p, int mask_id, hipStream_t stream) {
                                        dq_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
         bool small = false;
         constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DQ);
-        if constexpr (served) small = bwd_takes_small((long long)p.B * p.H, p.T, D, Elem<E>::kDType, CHILL_PASS_DQ);
+        if constexpr (served) small = bwd_takes_small(MASK_ID, (long long)p.B * p.H, p.T, D, Elem<E>::kDType, CHILL_PASS_DQ);
         bool regs2 = false;
         if constexpr (dq_regs2_is_optional(D, Elem<E>::kDType)) regs2 = dq_takes_regs2(MASK_ID, (long long)p.B * p.H, p.T);
         if (small) {
@@ -1396,7 +1407,7 @@ int launch_dkdv(const BwdParams& p, int mask_id, hipStream_t stream) {
                                        dkdv_tile_config(MASK_ID, D, Elem<E>::kDType, false).waves;
         bool small = false;
         constexpr bool served = bwd_small_serves(D, Elem<E>::kDType, CHILL_PASS_DKDV);
-        if constexpr (served) small = bwd_takes_small((long long)p.B * p.H_kv, p.T, D, Elem<E>::kDType, CHILL_PASS_DKDV);
+        if constexpr (served) small = bwd_takes_small(MASK_ID, (long long)p.B * p.H_kv, p.T, D, Elem<E>::kDType, CHILL_PASS_DKDV);
         bool regs = false;
         if constexpr (dkdv_regs_is_optional(D, Elem<E>::kDType))
             regs = dkdv_takes_regs(MASK_ID, p.margs.a0, mask_band_keys(MASK_ID, p.margs.a0, p.margs.a1), D, (long long)p.B * p.H_kv, p.T);

@@ -51,9 +51,12 @@ __device__ __forceinline__ void bwd_small_merge(const char* smem, int wave_bytes
 }
 
 // ------------------------------------------------------------------------------------------ dQ
-template <typename E, int D, int MASK>
-__global__ __launch_bounds__(kFwdSmallWaves * 64) void dq_small_kernel(BwdParams p, int n_q_tiles, int total_items,
-                                                                       int has_full_blocks) {
+// TILES = 2: a workgroup of eight waves takes two 32-row blocks side by side, block j from the long end and block j
+// from the short end of one head, four waves each with an LDS area of their own, as fwd_small_kernel does; the two
+// halves meet at the one barrier of the kernel and nowhere else.
+template <typename E, int D, int MASK, int TILES>
+__global__ __launch_bounds__(kFwdSmallWaves * 64 * TILES) void dq_small_kernel(BwdParams p, int n_q_tiles, int total_items,
+                                                                               int has_full_blocks) {
     using ET = typename Elem<E>::type;
     typedef LdsTile<E, D> L;
     constexpr int NW = kFwdSmallWaves;
@@ -61,17 +64,26 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void dq_small_kernel(BwdParams
     constexpr int DB = (D + 31) / 32;
     constexpr int TILE_BYTES = L::bytes(32);
     constexpr int WAVE_BYTES = bwd_small_wave_bytes(D, Elem<E>::kDType, 1);
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    extern __shared__ __attribute__((aligned(16))) char smem_all[];
 
     const int item = blockIdx.x;
     if (item >= total_items) return;
-    const int bh = item / n_q_tiles;
-    const int qt = n_q_tiles - 1 - item % n_q_tiles;  // last tiles first: under causal-like masks the longest
+    const int half = TILES == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / NT) : 0;  // which block of the workgroup
+    char* smem = smem_all + half * (NW * WAVE_BYTES);
+    // the blocks of all heads from the long end to the short end (under causal-like masks: longest first, so that a launch
+    // of more workgroups than fit at once ends without stragglers); pairs of blocks: all of the same length
+    const int per_head = TILES == 2 ? (n_q_tiles + 1) / 2 : n_q_tiles;
+    const int n_heads = total_items / per_head;
+    const int bh = item % n_heads;
+    const int j = item / n_heads;
+    const int qt = half == 0 ? n_q_tiles - 1 - j : j;
+    // (an odd number of blocks: the middle one has no partner)
+    const bool has_tile = half == 0 || n_q_tiles - 1 - j != j;
     const int b = bh / p.H;
     const int hd = bh % p.H;
     const int hkv = hd / p.group;
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x % NT;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;
@@ -82,13 +94,16 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void dq_small_kernel(BwdParams
 
     const int qb = qt * 32;
     ET* dqbase = reinterpret_cast<ET*>(p.dq) + b * p.sdq.b + hd * p.sdq.h;
-    if (qb >= seq_len) {
-        // rows at or beyond lens[b] receive 0 (the reference relies on the adapter's zero-fill, chill.py:292)
-        zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(32, p.T - qb), tid);
-        if (p.delta_out != nullptr) {
-            // (the dK/dV launch that follows reads delta of every row of the tiles it visits)
-            for (int i = tid; i < imin(32, p.T - qb); i += NT) p.delta_out[b * p.delta_b + hd * p.delta_h + qb + i] = 0.f;
+    if (!has_tile || qb >= seq_len) {
+        if (has_tile) {
+            // rows at or beyond lens[b] receive 0 (the reference relies on the adapter's zero-fill, chill.py:292)
+            zero_rows<E, D, NT>(dqbase, p.sdq.t, qb, imin(32, p.T - qb), tid);
+            if (p.delta_out != nullptr) {
+                // (the dK/dV launch that follows reads delta of every row of the tiles it visits)
+                for (int i = tid; i < imin(32, p.T - qb); i += NT) p.delta_out[b * p.delta_b + hd * p.delta_h + qb + i] = 0.f;
+            }
         }
+        if constexpr (TILES == 2) __syncthreads();  // the other half's one barrier
         return;
     }
 
@@ -194,8 +209,11 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void dkdv_small_kernel(BwdPara
 
     const int item = blockIdx.x;
     if (item >= total_items) return;
-    const int bh = item / n_k_tiles;
-    const int kt = item % n_k_tiles;  // first tiles first: under causal-like masks the longest
+    // the key blocks of all heads from the first to the last (under causal-like masks: longest first, so that a launch of
+    // more workgroups than fit at once ends without stragglers)
+    const int n_heads = total_items / n_k_tiles;
+    const int bh = item % n_heads;
+    const int kt = item / n_heads;
     const int b = bh / p.H_kv;
     const int hkv = bh % p.H_kv;
 

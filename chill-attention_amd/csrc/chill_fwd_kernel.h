@@ -498,17 +498,25 @@ int launch_fwd_shape(const FwdParams& p, hipStream_t stream) {
 // A launch far too small for the chip: 32 query rows per workgroup, the keys split over its waves.
 template <typename E, int D, int MASK_ID>
 int launch_fwd_small(const FwdParams& p, hipStream_t stream) {
-    constexpr int kLdsBytes = fwd_small_lds_bytes(D, Elem<E>::kDType);
+    constexpr int kLdsOne = fwd_small_lds_bytes(D, Elem<E>::kDType);
     const int n_q_tiles = cdiv(p.T, 32);
-    const int total = p.B * p.H * n_q_tiles;  // (at most kComputeUnits / 4 * 4 * 32 by fwd_takes_small)
-    void (*kern)(FwdParams, int, int, int) = fwd_small_kernel<E, D, MASK_ID>;
+    // (at most kComputeUnits / 4 * 4 * 32 q-tiles by fwd_takes_small)
+    bool two = false;
+    if constexpr (small_fits_two_tiles(kLdsOne)) two = small_takes_two_tiles((long long)p.B * p.H * n_q_tiles);
+    const int total = p.B * p.H * (two ? (n_q_tiles + 1) / 2 : n_q_tiles);
+    const int lds_bytes = two ? 2 * kLdsOne : kLdsOne;
+    void (*kern)(FwdParams, int, int, int) = fwd_small_kernel<E, D, MASK_ID, 1>;
+    if constexpr (small_fits_two_tiles(kLdsOne)) {
+        if (two) kern = fwd_small_kernel<E, D, MASK_ID, 2>;
+    }
     const bool hfb = Mask<MASK_ID>::has_full_blocks(32, 32, p.T, p.margs);
-    if (kLdsBytes > 48 * 1024) {
+    if (lds_bytes > 48 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kLdsBytes) != hipSuccess)
+                                lds_bytes) != hipSuccess)
             return CHILL_ERR_HIP;
     }
-    hipLaunchKernelGGL(kern, dim3(total), dim3(kFwdSmallWaves * 64), kLdsBytes, stream, p, n_q_tiles, total, hfb ? 1 : 0);
+    hipLaunchKernelGGL(kern, dim3(total), dim3(kFwdSmallWaves * 64 * (two ? 2 : 1)), lds_bytes, stream, p, n_q_tiles, total,
+                       hfb ? 1 : 0);
     return (hipGetLastError() == hipSuccess) ? CHILL_OK : CHILL_ERR_HIP;
 }
 
@@ -523,7 +531,7 @@ int launch_fwd(const FwdParams& p, int mask_id, hipStream_t stream) {
         constexpr bool has_short_row = fwd_tile_config(MASK_ID, D, Elem<E>::kDType, 1).waves !=
                                        fwd_tile_config(MASK_ID, D, Elem<E>::kDType).waves;
         bool small = false;
-        if constexpr (D * Elem<E>::kBytes <= 512) small = fwd_takes_small((long long)p.B * p.H, p.T, D, Elem<E>::kDType);
+        if constexpr (D * Elem<E>::kBytes <= 512) small = fwd_takes_small(MASK_ID, (long long)p.B * p.H, p.T, D, Elem<E>::kDType);
         if (small) {
             if constexpr (D * Elem<E>::kBytes <= 512) status = launch_fwd_small<E, D, MASK_ID>(p, stream);
         } else if constexpr (has_short_row) {

@@ -20,9 +20,14 @@ namespace chill {
 
 // (kFwdSmallWaves, fwd_small_lds_bytes and the launches that come here: chill_tiles.h)
 
-template <typename E, int D, int MASK>
-__global__ __launch_bounds__(kFwdSmallWaves * 64) void fwd_small_kernel(FwdParams p, int n_q_tiles, int total_items,
-                                                                        int has_full_blocks) {
+// TILES = 2: a workgroup of eight waves takes two q-tiles side by side, tile j from the end and tile j from the start of
+// one head, four waves each with an LDS area of their own.  Under causal-like masks the two add up to the same work
+// for every workgroup, where workgroups of one q-tile each leave the CUs that drew two long ones to finish alone
+// (taken when the launch has more workgroups than the chip has CUs: fwd_small_tiles).  The two halves meet at the
+// one barrier of the kernel and nowhere else.
+template <typename E, int D, int MASK, int TILES>
+__global__ __launch_bounds__(kFwdSmallWaves * 64 * TILES) void fwd_small_kernel(FwdParams p, int n_q_tiles, int total_items,
+                                                                                int has_full_blocks) {
     using ET = typename Elem<E>::type;
     using M = Mask<MASK>;
     typedef LdsTile<E, D> L;
@@ -33,17 +38,26 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void fwd_small_kernel(FwdParam
     // K block, V block (later the partial O^T); then m and l of the wave's lanes
     constexpr int WAVE_BYTES = fwd_small_wave_bytes(D, Elem<E>::kDType);
     constexpr int ML_OFF = WAVE_BYTES - 2 * 64 * 4;
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    extern __shared__ __attribute__((aligned(16))) char smem_all[];
 
     const int item = blockIdx.x;
     if (item >= total_items) return;
-    const int bh = item / n_q_tiles;
-    const int qt = n_q_tiles - 1 - item % n_q_tiles;  // last tiles first: under causal-like masks the longest
+    const int half = TILES == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / NT) : 0;  // which q-tile of the workgroup
+    char* smem = smem_all + half * (NW * WAVE_BYTES);
+    // the q-tiles of all heads from the last to the first (under causal-like masks: longest first, so that a launch of
+    // more workgroups than fit at once ends without stragglers); pairs of q-tiles: all of the same length
+    const int per_head = TILES == 2 ? (n_q_tiles + 1) / 2 : n_q_tiles;
+    const int n_heads = total_items / per_head;
+    const int bh = item % n_heads;
+    const int j = item / n_heads;
+    const int qt = half == 0 ? n_q_tiles - 1 - j : j;
+    // (an odd number of q-tiles: the middle one has no partner)
+    const bool has_tile = half == 0 || n_q_tiles - 1 - j != j;
     const int b = bh / p.H;
     const int hd = bh % p.H;
     const int hkv = hd / p.group;
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x % NT;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 31;
@@ -55,12 +69,15 @@ __global__ __launch_bounds__(kFwdSmallWaves * 64) void fwd_small_kernel(FwdParam
     const int qb = qt * 32;
     ET* obase = reinterpret_cast<ET*>(p.o) + b * p.so.b + hd * p.so.h;
     float* lse_base = p.lse ? p.lse + b * p.lse_b + hd * p.lse_h : nullptr;
-    if (qb >= seq_len) {
-        // nothing attends here: the output rows are defined to be zero (chill.py:96, chill_fwd.py:70-71)
-        const int nrows = imin(32, p.T - qb);
-        zero_rows<E, D, NT>(obase, p.so.t, qb, nrows, tid);
-        if (lse_base)
-            for (int i = tid; i < nrows; i += NT) lse_base[qb + i] = 0.f;
+    if (!has_tile || qb >= seq_len) {
+        if (has_tile) {
+            // nothing attends here: the output rows are defined to be zero (chill.py:96, chill_fwd.py:70-71)
+            const int nrows = imin(32, p.T - qb);
+            zero_rows<E, D, NT>(obase, p.so.t, qb, nrows, tid);
+            if (lse_base)
+                for (int i = tid; i < nrows; i += NT) lse_base[qb + i] = 0.f;
+        }
+        if constexpr (TILES == 2) __syncthreads();  // the other half's one barrier
         return;
     }
 

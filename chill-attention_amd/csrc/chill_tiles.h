@@ -149,9 +149,41 @@ constexpr int fwd_small_wave_bytes(int D, int dtype) {
     return (blocks > partial ? blocks : partial) + 2 * 64 * 4;
 }
 constexpr int fwd_small_lds_bytes(int D, int dtype) { return kFwdSmallWaves * fwd_small_wave_bytes(D, dtype); }
-constexpr bool fwd_takes_small(long long batch_heads, int T, int D, int dtype) {
+// fp32, whose ordinary kernels give a wave 32 rows and all their keys at 2 us and more per block, is served much
+// further up since the small kernels balance their launches (small_takes_two_tiles, below).  Measured against
+// fwd_kernel / dq_kernel / dkdv_kernel at head dims 32, 64 and 128, T = 512 .. 4096, 1536 .. 32768 tiles: under
+// masks whose rows grow with their index (causal, prefix-LM) the forward wins up to 2048 tiles (B1 H24 T2048 D64:
+// 300 -> 154 us; at 2048 tiles 373 -> 359, at 4096 +5 .. +9 %; head dim 128: 387 -> 317 at 1536 tiles, +11 .. +15 %
+// at 2048), dQ up to 8192 tiles (B1 H24 T2048: 406 -> 195 us; B4 H16 T4096: 2000 -> 1750; head dim 128: 3925 -> 3820),
+// dK/dV up to 4096 tiles at T <= 2048 (B4 H16 T2048: 797 -> 715 us; prefix-LM B8 H32 T1024, 8192 tiles: +9 %) and 1024
+// at T = 4096 (B1 H8: 523 -> 333 us; B1 H16: 606 -> 645); under the other masks, whose tiles are all alike, forward
+// and dQ win up to 1536 tiles (full mask B1 H24 T2048 D64: 318 -> 276 and 421 -> 337 us; sliding window 70 -> 60 and
+// 104 -> 85) and tie or lose from 2048 on, and dK/dV does not win beyond its 512.
+constexpr bool mask_rows_grow(int mask_id) { return mask_id == CHILL_MASK_CAUSAL || mask_id == CHILL_MASK_PREFIX_LM; }
+constexpr long long fwd_small_max_tiles(int mask_id, int D, int dtype) {
+    if (dtype != CHILL_F32) return (D >= 128 ? 2 : 1) * kComputeUnits;
+    return (mask_rows_grow(mask_id) && D <= 64 ? 8 : 6) * kComputeUnits;
+}
+constexpr bool fwd_takes_small(int mask_id, long long batch_heads, int T, int D, int dtype) {
     return CHILL_TUNE_FWD_SMALL && D * elem_bytes(dtype) <= 512 && T <= kFwdSmallMaxT &&
-           batch_heads * ((T + 31) / 32) <= ((dtype == CHILL_F32 || D >= 128) ? 2 : 1) * kComputeUnits;
+           batch_heads * ((T + 31) / 32) <= fwd_small_max_tiles(mask_id, D, dtype);
+}
+
+// With more 32-row tiles than the chip has CUs the workgroups of a launch no longer run all at once or alone on their
+// CUs, and under causal-like masks, where a tile's work grows with its index, the launch ends when the CU with the
+// longest tiles does.  Then, in the forward and dQ, a workgroup of eight waves takes two tiles side by side, tile j
+// from the end and tile j from the start of a head, which add up to the same work for every workgroup, where two areas
+// fit in LDS (the wave then has 256 registers: enough for the forward and dQ, not for dK/dV with K, V and two
+// accumulators); and every small launch takes its tiles longest first across all heads.  Measured on fp32 at head dim
+// 64, forward / dQ / dK/dV: prefix-LM B1 H8 T2048 83 / 127 / 161 -> 66 / 87 / 127 us, causal 81 / 126 / 159 ->
+// 52 / 69 / 97, causal B2 H8 T1024 45 / 71 / 90 -> 30 / 40 / 58; two tiles per workgroup against the new order
+// alone: forward 66 against 69, dQ 87 against 101 us on the prefix-LM shape.
+constexpr bool small_fits_two_tiles(int lds_bytes_one) { return 2 * lds_bytes_one <= 160 * 1024; }
+constexpr bool small_takes_two_tiles(long long tiles) { return tiles > kComputeUnits; }
+// what the report says of such a launch: 32 rows and 4 waves per tile; the LDS of the workgroup (of both tiles)
+constexpr TileConfig small_tile_config(int lds_bytes_one, long long tiles) {
+    return TileConfig{32, 32, kFwdSmallWaves,
+                      (small_fits_two_tiles(lds_bytes_one) && small_takes_two_tiles(tiles)) ? 2 * lds_bytes_one : lds_bytes_one};
 }
 
 // The backward of such launches (dq_small_kernel, dkdv_small_kernel): the same split of the streamed
@@ -176,10 +208,15 @@ constexpr int bwd_small_lds_bytes(int D, int dtype, int outputs) { return kFwdSm
 constexpr bool bwd_small_serves(int D, int dtype, int pass) {
     return CHILL_TUNE_BWD_SMALL && (pass == CHILL_PASS_DKDV ? D <= 64 : (D <= 128 && D * elem_bytes(dtype) <= 512));
 }
-constexpr bool bwd_takes_small(long long batch_heads, int T, int D, int dtype, int pass) {
-    const int chips = pass == CHILL_PASS_DKDV ? (dtype == CHILL_F32 ? 2 : 1) : ((dtype == CHILL_F32 || D <= 64) ? 2 : 1);
+// (fp32 beyond that: the measurements at fwd_small_max_tiles)
+constexpr long long bwd_small_max_tiles(int mask_id, int T, int D, int dtype, int pass) {
+    if (dtype != CHILL_F32) return ((pass == CHILL_PASS_DQ && D <= 64) ? 2 : 1) * kComputeUnits;
+    if (pass == CHILL_PASS_DQ) return (mask_rows_grow(mask_id) ? 32 : 6) * kComputeUnits;
+    return (mask_rows_grow(mask_id) ? (T <= 2048 ? 16 : 4) : 2) * kComputeUnits;
+}
+constexpr bool bwd_takes_small(int mask_id, long long batch_heads, int T, int D, int dtype, int pass) {
     return bwd_small_serves(D, dtype, pass) && T <= kFwdSmallMaxT * CHILL_TUNE_BWD_SMALL_SCALE &&
-           batch_heads * ((T + 31) / 32) <= (long long)chips * kComputeUnits * CHILL_TUNE_BWD_SMALL_SCALE;
+           batch_heads * ((T + 31) / 32) <= bwd_small_max_tiles(mask_id, T, D, dtype, pass) * CHILL_TUNE_BWD_SMALL_SCALE;
 }
 
 constexpr TileConfig fwd_tile_config(int mask_id, int D, int dtype, int T = kLongSequence) {
@@ -351,15 +388,15 @@ inline int tile_config(int mask_id, long long mask_arg0, long long band_keys, in
     if (D != 16 && D != 32 && D != 64 && D != 128 && D != 256) return CHILL_ERR_BAD_HEAD_DIM;
     switch (pass) {
         case CHILL_PASS_FWD:
-            if (T != kLongSequence && fwd_takes_small(batch_heads, T, D, dtype)) {
-                *out = TileConfig{32, 32, kFwdSmallWaves, fwd_small_lds_bytes(D, dtype)};
+            if (T != kLongSequence && fwd_takes_small(mask_id, batch_heads, T, D, dtype)) {
+                *out = small_tile_config(fwd_small_lds_bytes(D, dtype), batch_heads * ((T + 31) / 32));
                 return CHILL_OK;
             }
             *out = fwd_tile_config(mask_id, D, dtype, fwd_takes_short_row(mask_id, band_keys, batch_heads, T) ? 1 : kLongSequence);
             return CHILL_OK;
         case CHILL_PASS_DQ:
-            if (T != kLongSequence && bwd_takes_small(batch_heads, T, D, dtype, CHILL_PASS_DQ)) {
-                *out = TileConfig{32, 32, kFwdSmallWaves, bwd_small_lds_bytes(D, dtype, 1)};
+            if (T != kLongSequence && bwd_takes_small(mask_id, batch_heads, T, D, dtype, CHILL_PASS_DQ)) {
+                *out = small_tile_config(bwd_small_lds_bytes(D, dtype, 1), batch_heads * ((T + 31) / 32));
                 return CHILL_OK;
             }
             if (dq_regs2_is_optional(D, dtype) && (T == kLongSequence ? !mask_is_banded(mask_id) : dq_takes_regs2(mask_id, batch_heads, T))) {
@@ -370,7 +407,7 @@ inline int tile_config(int mask_id, long long mask_arg0, long long band_keys, in
             return CHILL_OK;
         case CHILL_PASS_DKDV:
             // (for this pass batch_heads counts the key / value heads)
-            if (T != kLongSequence && bwd_takes_small(batch_heads, T, D, dtype, CHILL_PASS_DKDV)) {
+            if (T != kLongSequence && bwd_takes_small(mask_id, batch_heads, T, D, dtype, CHILL_PASS_DKDV)) {
                 *out = TileConfig{32, 32, kFwdSmallWaves, bwd_small_lds_bytes(D, dtype, 2)};
                 return CHILL_OK;
             }

@@ -222,8 +222,10 @@ int chill_tile_config(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, i
  * the chip (the reference's tables, autotune.py:11-119, do not depend on the shape; its autotuner's key
  * does, autotune.py:129-240), and the dK/dV row one that covers half as many key rows for such grids
  * (batch_heads = B * H_kv for that pass).  Launches far too small for the chip (a few hundred 32-row
- * blocks in all) take kernels of their own, in which a workgroup owns 32 rows and its four waves split
- * the streamed axis: reported as {32, 32, 4, lds_bytes}.  chill_tile_config reports the row of long
+ * blocks in all; fp32, whose ordinary kernels are slow per block, up to a few thousand, depending on the
+ * mask) take kernels of their own, in which four waves own 32 rows and split the streamed axis: reported
+ * as {32, 32, 4, lds_bytes}, lds_bytes being the workgroup's, which in the forward and dQ holds two such
+ * blocks of eight waves in all when the launch has more blocks than the chip has CUs.  chill_tile_config reports the row of long
  * sequences on a full chip. */
 int chill_tile_config_for_shape(int32_t mask_id, int32_t D, int32_t dtype, int32_t pass, int64_t batch_heads,
                                 int32_t T, int32_t out[4]);

@@ -138,6 +138,30 @@ def test_tile_table():
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
     assert _lib.lib.chill_tile_config_for_shape(1, 128, _lib.BF16, 0, 1, 0, (ctypes.c_int32 * 4)()) == -8
+    # launches far too small for the chip: 32 rows per workgroup; fp32 much further up than 16-bit inputs, and furthest
+    # under masks whose rows grow with their index (tiles = B * H * T / 32)
+    prefix, full = ca.PrefixLMChillMask(100), ca.FullChillMask()
+    for mask, dt, D, p, bh, T, small in (
+            (causal, torch.bfloat16, 64, _lib.PASS_FWD, 8, 1024, True), (causal, torch.bfloat16, 64, _lib.PASS_FWD, 9, 1024, False),
+            (causal, torch.bfloat16, 128, _lib.PASS_FWD, 16, 1024, True), (causal, torch.bfloat16, 128, _lib.PASS_FWD, 17, 1024, False),
+            (causal, torch.float32, 64, _lib.PASS_FWD, 32, 2048, True), (causal, torch.float32, 64, _lib.PASS_FWD, 33, 2048, False),
+            (prefix, torch.float32, 128, _lib.PASS_FWD, 24, 2048, True), (prefix, torch.float32, 128, _lib.PASS_FWD, 25, 2048, False),
+            (full, torch.float32, 64, _lib.PASS_FWD, 24, 2048, True), (window, torch.float32, 64, _lib.PASS_FWD, 25, 2048, False),
+            (causal, torch.float32, 64, _lib.PASS_FWD, 1, 4097, False),
+            (causal, torch.float32, 64, _lib.PASS_DQ, 64, 4096, True), (causal, torch.float32, 128, _lib.PASS_DQ, 65, 4096, False),
+            (full, torch.float32, 64, _lib.PASS_DQ, 24, 2048, True), (full, torch.float32, 64, _lib.PASS_DQ, 25, 2048, False),
+            (causal, torch.float16, 64, _lib.PASS_DQ, 16, 1024, True), (causal, torch.float16, 128, _lib.PASS_DQ, 16, 1024, False),
+            (causal, torch.float32, 64, _lib.PASS_DKDV, 64, 2048, True), (causal, torch.float32, 64, _lib.PASS_DKDV, 65, 2048, False),
+            (prefix, torch.float32, 32, _lib.PASS_DKDV, 8, 4096, True), (prefix, torch.float32, 32, _lib.PASS_DKDV, 9, 4096, False),
+            (full, torch.float32, 64, _lib.PASS_DKDV, 8, 2048, True), (full, torch.float32, 64, _lib.PASS_DKDV, 9, 2048, False),
+            (causal, torch.float32, 128, _lib.PASS_DKDV, 1, 512, False), (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 8, 1024, True),
+            (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 9, 1024, False)):
+        c = tile_config(mask, D, dt, p, seq_len=T, batch_heads=bh)
+        assert (c["rows"] == 32 and c["streamed"] == 32) == small, (mask, dt, D, p, bh, T, c)
+    # (more tiles than CUs: forward and dQ workgroups hold two tiles where two LDS areas fit)
+    one = tile_config(causal, 64, torch.float32, _lib.PASS_FWD, seq_len=1024, batch_heads=8)["lds_bytes"]
+    assert tile_config(causal, 64, torch.float32, _lib.PASS_FWD, seq_len=1024, batch_heads=9)["lds_bytes"] == 2 * one
+    assert tile_config(causal, 128, torch.float32, _lib.PASS_FWD, seq_len=1024, batch_heads=9)["lds_bytes"] == 4 * (2 * 32 * 512 + 512)
     # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU (at head dim 64
     # for short sequences, small grids and banded masks; long sequences: K in registers, below)
     for D, T, rows, waves in ((64, 4095, 64, 4), (32, None, 64, 4), (32, 8192, 64, 4)):

@@ -202,6 +202,89 @@ def test_small_launch_backward(m, dtype):
                                        msg=lambda msg: f"{name} T={T} D={D}: {msg}")
 
 
+# Small launches of more 32-row tiles than the chip has CUs: forward and dQ workgroups of eight waves take two tiles side
+# by side (tile j from the end and tile j from the start of a head).  An even and an odd number of tiles per head (the
+# middle one has no partner), GQA, lens that leave one of the two tiles, or both, behind the end of the sequence.
+TWO_TILE_CASES = [
+    ("prefix-lm-f32-D64", torch.float32, 1, 8, 8, 2048, 64, ("PrefixLMChillMask", (1024,)), None),
+    ("causal-f32-D32-odd-lens", torch.float32, 3, 3, 3, 1500, 32, ("CausalChillMask", ()), (1500, 40, 777)),
+    ("causal-bf16-D128-gqa-odd-lens", torch.bfloat16, 2, 6, 2, 1111, 128, ("CausalChillMask", ()), (1111, 1)),
+    ("sliding-f16-D128-lens", torch.float16, 1, 5, 5, 2048, 128, ("SlidingWindowChillMask", (100, 7)), (1025,)),
+    ("chunkwise-f32-D16", torch.float32, 2, 4, 4, 1990, 16, ("ChunkwiseChillMask", (100, 1)), None),
+    ("full-f32-D64-gqa", torch.float32, 1, 12, 3, 1000, 64, ("FullChillMask", ()), (999,)),
+    # fp32 takes these kernels far beyond that: 2048 tiles under a causal mask in all three passes
+    ("causal-f32-D64-2048-tiles-lens", torch.float32, 2, 16, 16, 2048, 64, ("CausalChillMask", ()), (2048, 1500)),
+    # rows of 512 bytes: two areas do not fit in LDS, one tile per workgroup, longest first across the heads
+    ("prefix-lm-f32-D128-1536-tiles-gqa", torch.float32, 1, 24, 12, 2048, 128, ("PrefixLMChillMask", (300,)), None),
+]
+
+
+@pytest.mark.parametrize("case", TWO_TILE_CASES, ids=lambda c: c[0])
+def test_small_launch_with_two_tiles_per_workgroup(case):
+    """Forward (O and LSE2, chill_fwd.py:215-330) and backward (chill_bwd_dq.py:300-394, chill_bwd_dkdv.py:347-508) of
+    small launches whose forward and dQ workgroups hold two tiles (asserted from the tile report: 32 rows per tile,
+    twice the LDS of one tile), against the oracle."""
+    _, dtype, B, H, Hkv, T, D, m, lens = case
+    mask = make_mask(m)
+    for pass_id, heads, tiles in ((_lib.PASS_FWD, H, 2), (_lib.PASS_DQ, H, 2), (_lib.PASS_DKDV, Hkv, 1)):
+        cfg = tile_config(mask, D, dtype, pass_id, seq_len=T, batch_heads=B * heads)
+        if cfg["rows"] != 32:
+            # (only the forward of every case is meant to take the small kernel: at head dim 128 the 16-bit backward of
+            # these sizes takes ordinary kernels)
+            assert pass_id != _lib.PASS_FWD and (dtype != torch.float32 or pass_id == _lib.PASS_DKDV), f"pass {pass_id} served by {cfg}"
+            continue
+        single = tile_config(mask, D, dtype, pass_id, seq_len=32, batch_heads=1)
+        assert (cfg["waves"], cfg["streamed"]) == (4, 32) and single["rows"] == 32
+        if 2 * single["lds_bytes"] > 160 * 1024:
+            tiles = 1
+        assert cfg["lds_bytes"] == tiles * single["lds_bytes"], f"pass {pass_id}: {cfg} against {single}"
+    torch.manual_seed(stable_seed(case[0]))
+    q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
+    lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    dout = torch.randn(B, H, T, D, device=DEV, dtype=dtype)
+    out, lse = ca.chill_attention(q, k, v, mask=mask, lens=lens_t, return_lse=True)
+    out.backward(dout)
+    qf, kf, vf = (x.detach().float().clone().requires_grad_() for x in (q, k, v))
+    ref, res_mask = orc.reference_naive(m[0], m[1], qf, kf, vf, lens_t)
+    ref.backward(dout.float() * res_mask)
+    check_close(out.detach() * res_mask, ref.detach(), dtype, OUT_TOL[dtype], D, "O")
+    want_lse = orc.lse2_dense(m[0], m[1], q.detach(), k.detach(), lens_t)
+    seen = torch.isfinite(want_lse)
+    torch.testing.assert_close(lse[seen].double(), want_lse[seen], atol=1e-4 if dtype == torch.float32 else 2e-2, rtol=1e-4)
+    assert (lse[~seen] == (-math.inf if lens is None else lse[~seen])).all()
+    for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
+        assert torch.isfinite(got).all(), name
+        check_close(got, want, dtype, GRAD_TOL[dtype], D, name)
+    if lens is not None:
+        for b, n in enumerate(lens):
+            assert (out[b, :, n:] == 0).all() and (q.grad[b, :, n:] == 0).all() and (k.grad[b, :, n:] == 0).all()
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_fp32_beyond_the_small_launch_kernels(D):
+    """The ordinary fp32 kernels (a wave owns 32 rows and walks all their blocks), which fp32 launches of up to 4096 rows
+    leave to the small-launch kernels far up: sequences longer than that take them whatever the grid (asserted), against
+    the oracle; GQA, lens, a ragged end."""
+    T, B, H, Hkv = 4100, 2, 2, 1
+    lens = torch.tensor([T, 3000], dtype=torch.int32, device=DEV)
+    for m in (("CausalChillMask", ()), ("SlidingWindowChillMask", (300, 20)), ("PrefixLMChillMask", (1000,))):
+        mask = make_mask(m)
+        for pass_id, heads in ((_lib.PASS_FWD, H), (_lib.PASS_DQ, H), (_lib.PASS_DKDV, Hkv)):
+            cfg = tile_config(mask, D, torch.float32, pass_id, seq_len=T, batch_heads=B * heads)
+            assert cfg["rows"] == 128, f"pass {pass_id} served by {cfg}"
+        torch.manual_seed(stable_seed(m, D, "fp32 long"))
+        q, k, v = (make_qkv((B, h, T, D), torch.float32, False).requires_grad_() for h in (H, Hkv, Hkv))
+        dout = torch.randn(B, H, T, D, device=DEV)
+        out = ca.chill_attention(q, k, v, mask=mask, lens=lens)
+        out.backward(dout)
+        qf, kf, vf = (x.detach().clone().requires_grad_() for x in (q, k, v))
+        ref, res_mask = orc.reference_naive(m[0], m[1], qf, kf, vf, lens)
+        ref.backward(dout * res_mask)
+        check_close(out.detach() * res_mask, ref.detach(), torch.float32, OUT_TOL[torch.float32], D, f"O {m[0]}")
+        for name, got, want in (("dv", v.grad, vf.grad), ("dk", k.grad, kf.grad), ("dq", q.grad, qf.grad)):
+            check_close(got, want, torch.float32, GRAD_TOL[torch.float32], D, f"{name} {m[0]}")
+
+
 def test_cpp_operator_matches_python_operator():
     """Eager calls go through the operator registered from C++; the torch.library operators (what
     torch.compile sees) must give the same bits, forward and backward, on the same kernels."""
@@ -343,8 +426,9 @@ RAMP_CASES = [
     ("d32-bf16", torch.bfloat16, 32, 2, 8, 8, 1024, (128, 4), (0, 1), "all", None),
     ("d256-regs", torch.bfloat16, 256, 2, 8, 8, 2048, (128, 4), (0, 1), "all", None),
     ("d256-regs-f16", torch.float16, 256, 2, 8, 8, 2048, (128, 4), (0, 1, 7), "wave", None),
-    ("f32-d64", torch.float32, 64, 4, 8, 8, 1024, (128, 4), (0, 1), "all", None),
-    ("f32-d128", torch.float32, 128, 4, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    # (fp32: more than 2048 tiles of 32 rows, where the small-launch kernels stop)
+    ("f32-d64", torch.float32, 64, 8, 10, 10, 1024, (128, 4), (0, 1), "all", None),
+    ("f32-d128", torch.float32, 128, 8, 10, 10, 1024, (128, 4), (0, 1), "all", None),
     ("small-d64", torch.bfloat16, 64, 1, 2, 2, 1024, (32, 4), (0, 1), "all", None),
     ("small-d128-f16", torch.float16, 128, 1, 2, 2, 1024, (32, 4), (0, 1), "all", None),
     ("small-d256", torch.bfloat16, 256, 1, 2, 2, 1024, (32, 4), (0, 1), "all", None),
@@ -772,7 +856,7 @@ DQ_DELTA_CASES = [
     ("registers-128", torch.bfloat16, 128, 1, 16, 8, 8200, ("CausalChillMask", ()), (8111,), (256, 4, 32)),
     ("registers-256-f16", torch.float16, 256, 1, 8, 8, 1030, ("FullChillMask", ()), (700,), (128, 4, 32)),
     ("split-f32-256", torch.float32, 256, 1, 4, 2, 530, ("CausalChillMask", ()), (333,), None),
-    ("f32-64", torch.float32, 64, 2, 8, 8, 1500, ("ChunkwiseChillMask", (64, 2)), (1500, 65), (128, 4, 32)),
+    ("f32-64", torch.float32, 64, 4, 12, 12, 1500, ("ChunkwiseChillMask", (64, 2)), (1500, 65, 1, 777), (128, 4, 32)),
     ("small-launch", torch.bfloat16, 64, 1, 2, 1, 300, ("CausalChillMask", ()), (129,), (32, 4, 32)),
     ("small-launch-f32", torch.float32, 32, 1, 3, 3, 257, ("FullChillMask", ()), None, (32, 4, 32)),
 ]
