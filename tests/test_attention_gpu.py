@@ -216,6 +216,9 @@ TWO_TILE_CASES = [
     ("causal-f32-D64-2048-tiles-lens", torch.float32, 2, 16, 16, 2048, 64, ("CausalChillMask", ()), (2048, 1500)),
     # rows of 512 bytes: two areas do not fit in LDS, one tile per workgroup, longest first across the heads
     ("prefix-lm-f32-D128-1536-tiles-gqa", torch.float32, 1, 24, 12, 2048, 128, ("PrefixLMChillMask", (300,)), None),
+    # a few fp32 heads of a long sequence
+    ("causal-f32-D64-T8192-gqa-lens", torch.float32, 1, 2, 1, 8192, 64, ("CausalChillMask", ()), (8000,)),
+    ("full-f32-D128-T8200", torch.float32, 1, 2, 2, 8200, 128, ("FullChillMask", ()), None),
 ]
 
 
@@ -262,12 +265,13 @@ def test_small_launch_with_two_tiles_per_workgroup(case):
 
 @pytest.mark.parametrize("D", [32, 64, 128])
 def test_fp32_beyond_the_small_launch_kernels(D):
-    """The ordinary fp32 kernels (a wave owns 32 rows and walks all their blocks), which fp32 launches of up to 4096 rows
-    leave to the small-launch kernels far up: sequences longer than that take them whatever the grid (asserted), against
-    the oracle; GQA, lens, a ragged end."""
-    T, B, H, Hkv = 4100, 2, 2, 1
-    lens = torch.tensor([T, 3000], dtype=torch.int32, device=DEV)
-    for m in (("CausalChillMask", ()), ("SlidingWindowChillMask", (300, 20)), ("PrefixLMChillMask", (1000,))):
+    """The ordinary fp32 kernels (a wave owns 32 rows and walks all their blocks), which fp32 launches leave to the
+    small-launch kernels up to thousands of 32-row tiles: grids beyond those limits (route asserted), against the oracle;
+    GQA, lens, a ragged end."""
+    for m, T, B, H, Hkv, lens in ((("CausalChillMask", ()), 4100, 4, 16, 8, (4100, 3000, 77, 4099)),
+                                  (("SlidingWindowChillMask", (300, 20)), 2100, 2, 12, 6, (2100, 1000)),
+                                  (("PrefixLMChillMask", (1000,)), 4100, 4, 16, 16, None)):
+        lens = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
         mask = make_mask(m)
         for pass_id, heads in ((_lib.PASS_FWD, H), (_lib.PASS_DQ, H), (_lib.PASS_DKDV, Hkv)):
             cfg = tile_config(mask, D, torch.float32, pass_id, seq_len=T, batch_heads=B * heads)
