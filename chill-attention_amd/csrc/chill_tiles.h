@@ -136,16 +136,17 @@ constexpr bool fwd_uses_regs(int D, int dtype) { return dtype != CHILL_F32 && D 
 // Forward launches far too small for the chip (fwd_small_kernel): a workgroup of four waves owns 32
 // query rows and its waves split the keys.  Per wave LDS holds a 32-row K block, a 32-row V block and
 // the wave's running max and row sum; rows of at most 512 bytes, so that four such areas fit.
-// It is taken while its grid of B * H * T / 32 workgroups is about what the chip holds at once
-// (measured against the ordinary forward, causal and full masks, T = 128 .. 4096, 1 .. 128 heads: with
-// up to 256 workgroups it wins everywhere, by 1.1x .. 1.5x for 16-bit inputs and up to 3.6x for fp32; with
-// 512 it still wins for fp32 and at head dim 128, where a block is more work, and loses 10-20 % at
-// head dim 64 and below; with 1024 it loses or ties).
+// For 16-bit inputs it is taken while its grid of B * H * T / 32 tiles is about what the chip holds at once
+// (measured against the ordinary forward, causal and full masks, T = 128 .. 16384, 1 .. 128 heads: with up to
+// 256 tiles it wins everywhere, by 1.1x .. 1.5x; with 512 it still wins at head dim 128, where a block is more
+// work, and under causal-like masks; with 1024 it loses or ties); fp32 much further up (fwd_small_max_tiles).
 constexpr int kFwdSmallWaves = 4;
-constexpr int kFwdSmallMaxT = 4096;
-// (fp32: measured up to 16384 rows; causal B1 H2 T8192 D64 forward 633 -> 193 us, dQ 883 -> 244, dK/dV 1032 -> 332, full
-// mask 645 -> 340, 908 -> 408, 1047 -> 597; causal B1 H4 T16384 forward 1318 -> 1224, dQ 2800 -> 1570)
-constexpr int small_max_rows(int dtype) { return dtype == CHILL_F32 ? 4 * kFwdSmallMaxT : kFwdSmallMaxT; }
+// (sequences of up to 16384 rows: with a head or two of such a sequence the ordinary kernels have a few dozen workgroups.
+// Measured at T = 8192: fp32 causal B1 H2 D64 forward 633 -> 193 us, dQ 883 -> 244, dK/dV 1032 -> 332, full mask
+// 645 -> 340, 908 -> 408, 1047 -> 597; fp32 causal B1 H4 T16384 forward 1318 -> 1224, dQ 2800 -> 1570; bf16 causal
+// B1 H2 D128 forward 142 -> 89, dQ 153 -> 90, full mask 145 -> 125 and 156 -> 132; bf16 causal B1 H1 D64 dQ 108 -> 54,
+// dK/dV 110 -> 76)
+constexpr int kFwdSmallMaxT = 16384;
 // (at the end the area also takes the wave's partial O^T, 4 KiB per 32 columns of the head dim)
 constexpr int fwd_small_wave_bytes(int D, int dtype) {
     const int blocks = 2 * 32 * D * elem_bytes(dtype), partial = ((D + 31) / 32) * 16 * 64 * 4;
@@ -164,11 +165,12 @@ constexpr int fwd_small_lds_bytes(int D, int dtype) { return kFwdSmallWaves * fw
 // 104 -> 85) and tie or lose from 2048 on, and dK/dV does not win beyond its 512.
 constexpr bool mask_rows_grow(int mask_id) { return mask_id == CHILL_MASK_CAUSAL || mask_id == CHILL_MASK_PREFIX_LM; }
 constexpr long long fwd_small_max_tiles(int mask_id, int D, int dtype) {
-    if (dtype != CHILL_F32) return (D >= 128 ? 2 : 1) * kComputeUnits;
+    // (16-bit head dims <= 64 at 512 tiles: causal B1 H2 T8192 69 -> 57 us, B1 H4 T4096 38 -> 31; full mask 71 -> 81, 39 -> 42)
+    if (dtype != CHILL_F32) return ((D >= 128 || mask_rows_grow(mask_id)) ? 2 : 1) * kComputeUnits;
     return (mask_rows_grow(mask_id) && D <= 64 ? 8 : 6) * kComputeUnits;
 }
 constexpr bool fwd_takes_small(int mask_id, long long batch_heads, int T, int D, int dtype) {
-    return CHILL_TUNE_FWD_SMALL && D * elem_bytes(dtype) <= 512 && T <= small_max_rows(dtype) &&
+    return CHILL_TUNE_FWD_SMALL && D * elem_bytes(dtype) <= 512 && T <= kFwdSmallMaxT &&
            batch_heads * ((T + 31) / 32) <= fwd_small_max_tiles(mask_id, D, dtype);
 }
 
@@ -213,12 +215,16 @@ constexpr bool bwd_small_serves(int D, int dtype, int pass) {
 }
 // (fp32 beyond that: the measurements at fwd_small_max_tiles)
 constexpr long long bwd_small_max_tiles(int mask_id, int T, int D, int dtype, int pass) {
-    if (dtype != CHILL_F32) return ((pass == CHILL_PASS_DQ && D <= 64) ? 2 : 1) * kComputeUnits;
+    // (16-bit dQ at 512 tiles, head dim 128: causal B1 H2 T8192 153 -> 90 us, B1 H4 T4096 82 -> 50, B1 H16 T1024 27 -> 23, full
+    // mask 156 -> 132 and 95 -> 75; at 1024 tiles wins and losses of up to 25 % either way)
+    // (16-bit dK/dV at 512 tiles, head dim 64, causal: B1 H2 T8192 118 -> 90 us, B1 H4 T4096 62 -> 52, B1 H16 T1024 20 -> 22; full
+    // mask 134 -> 164 and 76 -> 91)
+    if (dtype != CHILL_F32) return ((pass == CHILL_PASS_DQ || (mask_rows_grow(mask_id) && T >= 4096)) ? 2 : 1) * kComputeUnits;
     if (pass == CHILL_PASS_DQ) return (mask_rows_grow(mask_id) ? 32 : 6) * kComputeUnits;
     return (mask_rows_grow(mask_id) ? (T <= 2048 ? 16 : 4) : 2) * kComputeUnits;
 }
 constexpr bool bwd_takes_small(int mask_id, long long batch_heads, int T, int D, int dtype, int pass) {
-    return bwd_small_serves(D, dtype, pass) && T <= small_max_rows(dtype) * CHILL_TUNE_BWD_SMALL_SCALE &&
+    return bwd_small_serves(D, dtype, pass) && T <= kFwdSmallMaxT * CHILL_TUNE_BWD_SMALL_SCALE &&
            batch_heads * ((T + 31) / 32) <= bwd_small_max_tiles(mask_id, T, D, dtype, pass) * CHILL_TUNE_BWD_SMALL_SCALE;
 }
 

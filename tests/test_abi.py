@@ -142,22 +142,25 @@ def test_tile_table():
     # under masks whose rows grow with their index (tiles = B * H * T / 32)
     prefix, full = ca.PrefixLMChillMask(100), ca.FullChillMask()
     for mask, dt, D, p, bh, T, small in (
-            (causal, torch.bfloat16, 64, _lib.PASS_FWD, 8, 1024, True), (causal, torch.bfloat16, 64, _lib.PASS_FWD, 9, 1024, False),
+            (full, torch.bfloat16, 64, _lib.PASS_FWD, 8, 1024, True), (full, torch.bfloat16, 64, _lib.PASS_FWD, 9, 1024, False),
+            (causal, torch.bfloat16, 64, _lib.PASS_FWD, 16, 1024, True), (prefix, torch.float16, 32, _lib.PASS_FWD, 17, 1024, False),
             (causal, torch.bfloat16, 128, _lib.PASS_FWD, 16, 1024, True), (causal, torch.bfloat16, 128, _lib.PASS_FWD, 17, 1024, False),
             (causal, torch.float32, 64, _lib.PASS_FWD, 32, 2048, True), (causal, torch.float32, 64, _lib.PASS_FWD, 33, 2048, False),
             (prefix, torch.float32, 128, _lib.PASS_FWD, 24, 2048, True), (prefix, torch.float32, 128, _lib.PASS_FWD, 25, 2048, False),
             (full, torch.float32, 64, _lib.PASS_FWD, 24, 2048, True), (window, torch.float32, 64, _lib.PASS_FWD, 25, 2048, False),
             (causal, torch.float32, 64, _lib.PASS_FWD, 1, 16384, True), (causal, torch.float32, 64, _lib.PASS_FWD, 1, 16385, False),
-            (causal, torch.bfloat16, 64, _lib.PASS_FWD, 1, 4096, True), (causal, torch.bfloat16, 64, _lib.PASS_FWD, 1, 4097, False),
+            (causal, torch.bfloat16, 64, _lib.PASS_FWD, 1, 16384, True), (causal, torch.bfloat16, 64, _lib.PASS_FWD, 1, 16385, False),
             (full, torch.float32, 128, _lib.PASS_DQ, 2, 8192, True), (full, torch.float32, 64, _lib.PASS_DKDV, 2, 8192, True),
             (causal, torch.float32, 64, _lib.PASS_DQ, 64, 4096, True), (causal, torch.float32, 128, _lib.PASS_DQ, 65, 4096, False),
             (full, torch.float32, 64, _lib.PASS_DQ, 24, 2048, True), (full, torch.float32, 64, _lib.PASS_DQ, 25, 2048, False),
-            (causal, torch.float16, 64, _lib.PASS_DQ, 16, 1024, True), (causal, torch.float16, 128, _lib.PASS_DQ, 16, 1024, False),
+            (causal, torch.float16, 64, _lib.PASS_DQ, 16, 1024, True), (full, torch.float16, 128, _lib.PASS_DQ, 16, 1024, True),
+            (causal, torch.float16, 128, _lib.PASS_DQ, 17, 1024, False), (window, torch.float16, 128, _lib.PASS_DQ, 2, 8192, True),
             (causal, torch.float32, 64, _lib.PASS_DKDV, 64, 2048, True), (causal, torch.float32, 64, _lib.PASS_DKDV, 65, 2048, False),
             (prefix, torch.float32, 32, _lib.PASS_DKDV, 8, 4096, True), (prefix, torch.float32, 32, _lib.PASS_DKDV, 9, 4096, False),
             (full, torch.float32, 64, _lib.PASS_DKDV, 8, 2048, True), (full, torch.float32, 64, _lib.PASS_DKDV, 9, 2048, False),
             (causal, torch.float32, 128, _lib.PASS_DKDV, 1, 512, False), (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 8, 1024, True),
-            (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 9, 1024, False)):
+            (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 9, 1024, False), (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 4, 4096, True),
+            (full, torch.bfloat16, 64, _lib.PASS_DKDV, 4, 4096, False), (causal, torch.bfloat16, 64, _lib.PASS_DKDV, 5, 4096, False)):
         c = tile_config(mask, D, dt, p, seq_len=T, batch_heads=bh)
         assert (c["rows"] == 32 and c["streamed"] == 32) == small, (mask, dt, D, p, bh, T, c)
     # (more tiles than CUs: forward and dQ workgroups hold two tiles where two LDS areas fit)

@@ -219,6 +219,9 @@ TWO_TILE_CASES = [
     # a few fp32 heads of a long sequence
     ("causal-f32-D64-T8192-gqa-lens", torch.float32, 1, 2, 1, 8192, 64, ("CausalChillMask", ()), (8000,)),
     ("full-f32-D128-T8200", torch.float32, 1, 2, 2, 8200, 128, ("FullChillMask", ()), None),
+    # the same with 16-bit inputs: 512 tiles under a causal mask (at head dim 64 all three passes)
+    ("causal-bf16-D64-T8192", torch.bfloat16, 1, 2, 2, 8192, 64, ("CausalChillMask", ()), None),
+    ("prefix-lm-f16-D128-T16384-lens", torch.float16, 1, 1, 1, 16384, 128, ("PrefixLMChillMask", (5000,)), (16001,)),
 ]
 
 
@@ -419,15 +422,15 @@ RAMP_CASES = [
     ("d128-loop-paired-step-f16", torch.float16, 128, 4, 16, 8, 2048, (256, 8), (0, 1), "step-low", (2048, 1500, 300, 2047)),
     ("d128-loop-unpaired-step", torch.bfloat16, 128, 2, 8, 8, 2048, (256, 8), (0, 1), "step-wave", None),
     ("d64-loop-step", torch.bfloat16, 64, 8, 16, 16, 2048, (128, 4), (0, 1, 7), "step-low", None),
-    ("d64-loop-step-f16", torch.float16, 64, 2, 8, 4, 1024, (128, 4), (0, 1), "step", None),
-    ("d64-loop", torch.bfloat16, 64, 2, 8, 8, 1024, (128, 4), (0, 1, 4), "all", None),
-    ("d64-loop-f16", torch.float16, 64, 2, 8, 4, 1024, (128, 4), (0, 1, 4), "all", None),
+    ("d64-loop-step-f16", torch.float16, 64, 3, 8, 4, 1024, (128, 4), (0, 1), "step", None),
+    ("d64-loop", torch.bfloat16, 64, 3, 8, 8, 1024, (128, 4), (0, 1, 4), "all", None),
+    ("d64-loop-f16", torch.float16, 64, 3, 8, 4, 1024, (128, 4), (0, 1, 4), "all", None),
     ("d64-loop-paired-second-only", torch.float16, 64, 8, 16, 16, 2048, (128, 4), (0, 1, 7), "low", None),
     ("d64-loop-paired-lens", torch.bfloat16, 64, 8, 16, 16, 2048, (128, 4), (1, 7), "wave", (2048, 3, 999, 1024, 2048, 1500, 64, 129)),
     ("d128-short-row", torch.bfloat16, 128, 8, 8, 8, 1024, (128, 4), (0, 1), "all", None),
     ("d128-short-row-f16", torch.float16, 128, 8, 8, 8, 1024, (128, 4), (0, 1, 4), "wave", None),
-    ("d32", torch.float16, 32, 2, 8, 8, 1024, (128, 4), (0, 1), "all", None),
-    ("d32-bf16", torch.bfloat16, 32, 2, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("d32", torch.float16, 32, 3, 8, 8, 1024, (128, 4), (0, 1), "all", None),
+    ("d32-bf16", torch.bfloat16, 32, 3, 8, 8, 1024, (128, 4), (0, 1), "all", None),
     ("d256-regs", torch.bfloat16, 256, 2, 8, 8, 2048, (128, 4), (0, 1), "all", None),
     ("d256-regs-f16", torch.float16, 256, 2, 8, 8, 2048, (128, 4), (0, 1, 7), "wave", None),
     # (fp32: more than 2048 tiles of 32 rows, where the small-launch kernels stop)
