@@ -158,7 +158,7 @@ constexpr int fwd_small_lds_bytes(int D, int dtype) { return kFwdSmallWaves * fw
 // fwd_kernel / dq_kernel / dkdv_kernel at head dims 32, 64 and 128, T = 512 .. 4096, 1536 .. 32768 tiles: under
 // masks whose rows grow with their index (causal, prefix-LM) the forward wins up to 2048 tiles (B1 H24 T2048 D64:
 // 300 -> 154 us; at 2048 tiles 373 -> 359, at 4096 +5 .. +9 %; head dim 128: 387 -> 317 at 1536 tiles, +11 .. +15 %
-// at 2048), dQ up to 8192 tiles (B1 H24 T2048: 406 -> 195 us; B4 H16 T4096: 2000 -> 1750; head dim 128: 3925 -> 3820),
+// at 2048), dQ up to 16384 tiles (8192 at head dim 128; B1 H24 T2048: 406 -> 195 us; B4 H16 T4096: 2000 -> 1750; head dim 128: 3925 -> 3820),
 // dK/dV up to 4096 tiles at T <= 2048 (B4 H16 T2048: 797 -> 715 us; prefix-LM B8 H32 T1024, 8192 tiles: +9 %) and 1024
 // at T = 4096 (B1 H8: 523 -> 333 us; B1 H16: 606 -> 645); under the other masks, whose tiles are all alike, forward
 // and dQ win up to 1536 tiles (full mask B1 H24 T2048 D64: 318 -> 276 and 421 -> 337 us; sliding window 70 -> 60 and
@@ -220,7 +220,8 @@ constexpr long long bwd_small_max_tiles(int mask_id, int T, int D, int dtype, in
     // (16-bit dK/dV at 512 tiles, head dim 64, causal: B1 H2 T8192 118 -> 90 us, B1 H4 T4096 62 -> 52, B1 H16 T1024 20 -> 22; full
     // mask 134 -> 164 and 76 -> 91)
     if (dtype != CHILL_F32) return ((pass == CHILL_PASS_DQ || (mask_rows_grow(mask_id) && T >= 4096)) ? 2 : 1) * kComputeUnits;
-    if (pass == CHILL_PASS_DQ) return (mask_rows_grow(mask_id) ? 32 : 6) * kComputeUnits;
+    // (dQ at 16384 tiles, causal B8 H16 T4096: head dim 64 3775 -> 3393 us, 32 2045 -> 1901, 128 7822 -> 7909; at 32768 +1 .. +14 %)
+    if (pass == CHILL_PASS_DQ) return (mask_rows_grow(mask_id) ? (D <= 64 ? 64 : 32) : 6) * kComputeUnits;
     return (mask_rows_grow(mask_id) ? (T <= 2048 ? 16 : 4) : 2) * kComputeUnits;
 }
 constexpr bool bwd_takes_small(int mask_id, long long batch_heads, int T, int D, int dtype, int pass) {

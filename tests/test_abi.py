@@ -151,7 +151,8 @@ def test_tile_table():
             (causal, torch.float32, 64, _lib.PASS_FWD, 1, 16384, True), (causal, torch.float32, 64, _lib.PASS_FWD, 1, 16385, False),
             (causal, torch.bfloat16, 64, _lib.PASS_FWD, 1, 16384, True), (causal, torch.bfloat16, 64, _lib.PASS_FWD, 1, 16385, False),
             (full, torch.float32, 128, _lib.PASS_DQ, 2, 8192, True), (full, torch.float32, 64, _lib.PASS_DKDV, 2, 8192, True),
-            (causal, torch.float32, 64, _lib.PASS_DQ, 64, 4096, True), (causal, torch.float32, 128, _lib.PASS_DQ, 65, 4096, False),
+            (causal, torch.float32, 64, _lib.PASS_DQ, 128, 4096, True), (causal, torch.float32, 32, _lib.PASS_DQ, 129, 4096, False),
+            (causal, torch.float32, 128, _lib.PASS_DQ, 64, 4096, True), (causal, torch.float32, 128, _lib.PASS_DQ, 65, 4096, False),
             (full, torch.float32, 64, _lib.PASS_DQ, 24, 2048, True), (full, torch.float32, 64, _lib.PASS_DQ, 25, 2048, False),
             (causal, torch.float16, 64, _lib.PASS_DQ, 16, 1024, True), (full, torch.float16, 128, _lib.PASS_DQ, 16, 1024, True),
             (causal, torch.float16, 128, _lib.PASS_DQ, 17, 1024, False), (window, torch.float16, 128, _lib.PASS_DQ, 2, 8192, True),

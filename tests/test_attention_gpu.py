@@ -271,9 +271,9 @@ def test_fp32_beyond_the_small_launch_kernels(D):
     """The ordinary fp32 kernels (a wave owns 32 rows and walks all their blocks), which fp32 launches leave to the
     small-launch kernels up to thousands of 32-row tiles: grids beyond those limits (route asserted), against the oracle;
     GQA, lens, a ragged end."""
-    for m, T, B, H, Hkv, lens in ((("CausalChillMask", ()), 4100, 4, 16, 8, (4100, 3000, 77, 4099)),
+    for m, T, B, H, Hkv, lens in ((("CausalChillMask", ()), 4100, 8, 16, 8, (4100, 3000, 77, 4099, 1, 4100, 2222, 4000)),
                                   (("SlidingWindowChillMask", (300, 20)), 2100, 2, 12, 6, (2100, 1000)),
-                                  (("PrefixLMChillMask", (1000,)), 4100, 4, 16, 16, None)):
+                                  (("PrefixLMChillMask", (1000,)), 4100, 8, 16, 16, None)):
         lens = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
         mask = make_mask(m)
         for pass_id, heads in ((_lib.PASS_FWD, H), (_lib.PASS_DQ, H), (_lib.PASS_DKDV, Hkv)):
