@@ -134,7 +134,7 @@ void dq_kernel(BwdParams p, int n_q_tiles, int total_items,
     static_assert(NS == 2 || NS == 3, "two or three LDS stages");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
-    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    const int item = xcd_contiguous_item(blockIdx.x, total_items, dq_waves_per_simd<E, D, NW, TK, NS>());
     if (item < 0) return;
     const int bh = item / n_q_tiles;
     const int qt = n_q_tiles - 1 - item % n_q_tiles;
@@ -710,7 +710,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(NW == 4
     // table allocates the larger of the two needs)
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
-    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    // (the 64-row workgroups of head dims up to 64 run three to a CU)
+    const int item = xcd_contiguous_item(blockIdx.x, total_items, (NW == 4 && D <= 64) ? 3 : 1);
     if (item < 0) return;
     const int bh = item / n_k_tiles;
     // key tiles first-to-last: for causal-like masks the longest run first

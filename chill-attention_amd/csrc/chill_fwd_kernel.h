@@ -435,7 +435,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(fwd_wav
 void fwd_kernel(FwdParams p, int n_q_tiles, int total_items,
                                                       int wave_has_full_blocks, int paired) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int item = xcd_contiguous_item(blockIdx.x, total_items);
+    // (unpaired q-tiles differ in length: the order for a grid that is resident at once)
+    const int item = xcd_contiguous_item(blockIdx.x, total_items, paired ? 1 : fwd_waves_per_simd<E, D, NW, TK, NS>());
     if (item < 0) return;
     // paired: a workgroup takes q-tile j from the end and q-tile j from the start (equal work under
     // causal-like masks); unpaired: one q-tile per workgroup, last tiles first

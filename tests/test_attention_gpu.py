@@ -641,7 +641,19 @@ def _random_long_cases(n, seed):
     return cases
 
 
-@pytest.mark.parametrize("case", _random_long_cases(32, 20240607), ids=lambda c: c[0])
+# Grids of more workgroups than CUs that the chip still holds at once (two or three workgroups of four waves per CU):
+# the kernels take every second pass over an XCD's CUs in reverse order.  Totals that are no multiple of 8 or 32, a last
+# pass that is not full, GQA, lens.
+RESIDENT_GRID_CASES = [
+    ("resident-dq-330", 128, torch.bfloat16, 1, 10, 5, 4200, ("CausalChillMask", ()), None),
+    ("resident-dq-480-f16", 128, torch.float16, 3, 5, 5, 4096, ("PrefixLMChillMask", (700,)), (4096, 4000, 2000)),
+    ("resident-d64-297", 64, torch.bfloat16, 1, 9, 3, 4100, ("CausalChillMask", ()), (4001,)),
+    ("resident-d64-dkdv-650-f16", 64, torch.float16, 2, 10, 5, 4100, ("CausalChillMask", ()), None),
+    ("resident-d64-512", 64, torch.bfloat16, 1, 16, 16, 4096, ("SlidingWindowChillMask", (2000, 100)), None),
+]
+
+
+@pytest.mark.parametrize("case", _random_long_cases(32, 20240607) + RESIDENT_GRID_CASES, ids=lambda c: c[0])
 def test_random_long_sequences(case):
     """Forward and backward against the dense reference (chill_fwd.py:215-330, chill_bwd_dq.py:300-394,
     chill_bwd_dkdv.py:347-508 are what they must equal) on seeded random draws of long shapes."""
