@@ -75,6 +75,7 @@ def load_library(path: str) -> ctypes.CDLL:
         "chill_tile_config": (c_int32, [c_int32, c_int32, c_int32, c_int32, P(c_int32)]),
         "chill_tile_config_for_shape": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, P(c_int32)]),
         "chill_tile_config_for_launch": (c_int32, [P(ChillMaskDesc), c_int32, c_int32, c_int32, c_int64, c_int32, P(c_int32)]),
+        "chill_work_item": (c_int32, [c_int32, c_int32, c_int32]),
         "chill_mask_nnz": (c_int64, [MD, c_int32]),
         "chill_status_string": (c_char_p, [c_int32]),
         "chill_abi_version": (c_int32, []),
@@ -95,7 +96,7 @@ EXPORTED_SYMBOLS = (
     "chill_fwd", "chill_bwd_delta", "chill_bwd_dq", "chill_bwd_dq_delta", "chill_bwd_dkdv", "chill_bwd_noalloc", "chill_mask_eval_device",
     "chill_tile_ranges_device", "chill_mask_eval", "chill_mask_limits", "chill_tile_ranges",
     "chill_mask_is_full_block", "chill_mask_has_full_blocks", "chill_tile_config", "chill_tile_config_for_shape",
-    "chill_tile_config_for_launch",
+    "chill_tile_config_for_launch", "chill_work_item",
     "chill_mask_nnz",
     "chill_status_string", "chill_abi_version", "chill_has_user_mask",
 )

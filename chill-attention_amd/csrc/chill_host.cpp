@@ -150,6 +150,11 @@ int chill_tile_config_for_launch(const ChillMaskDesc* mask, int32_t D, int32_t d
     return report_tile_config(mask->id, a.a0, mask_band_keys(mask->id, a.a0, a.a1), D, dtype, pass, batch_heads, T, out);
 }
 
+int chill_work_item(int32_t workgroup, int32_t total, int32_t resident) {
+    if (workgroup < 0 || total < 1 || resident < 1) return CHILL_ERR_BAD_ARGUMENT;
+    return xcd_contiguous_item(workgroup, total, resident);
+}
+
 const char* chill_status_string(int32_t status) {
     switch (status) {
         case CHILL_OK: return "ok";

@@ -430,4 +430,34 @@ inline int tile_config(int mask_id, long long mask_arg0, long long band_keys, in
     }
 }
 
+// Work-item order: workgroups are dealt round-robin to the 8 XCDs (each with its own L2), so the
+// linear workgroup id is remapped to give every XCD a contiguous run of work items.  Returns the
+// work item index or -1 when this workgroup has nothing to do.
+//
+// `resident` = workgroups of the kernel that share a CU.  A grid that the chip holds at once (more workgroups than CUs,
+// at most `resident` per CU) is placed statically: the dispatcher deals an XCD's workgroups to its 32 CUs pass after
+// pass in the same CU order, so workgroup l of an XCD and workgroup l + 32 share a CU.  The kernels order their
+// work items longest first (under causal-like masks a tile's work grows with its index), which would hand a CU the
+// longest items of both passes and another the shortest; every second pass is therefore taken in reverse, and the two
+// items of a CU add up alike (measured on dq_kernel, 512 workgroups of four waves, causal bf16 at head dim 128:
+// B1 H16 T4096 148 -> 113 us, B1 H32 T2048 82 -> 66, B2 H8 T4096 147 -> 116, B1 H8 T8192 216 -> 204).  Larger grids
+// are dealt out as CUs become free, and longest first is the right order for that.
+CHILL_HD int xcd_contiguous_item(int wg, int total, int resident = 1) {
+    constexpr int kXcds = 8, kCusPerXcd = 32;
+    const int per = (total + kXcds - 1) / kXcds;
+    const int first = (wg % kXcds) * per;
+    int local = wg / kXcds;
+    if (resident > 1 && total > kXcds * kCusPerXcd && total <= resident * kXcds * kCusPerXcd) {
+        const int pass = local / kCusPerXcd;
+        if (pass & 1) {
+            const int valid = total - first < per ? total - first : per;  // items of this XCD
+            const int len = valid - pass * kCusPerXcd < kCusPerXcd ? valid - pass * kCusPerXcd : kCusPerXcd;
+            const int c = local - pass * kCusPerXcd;
+            if (c < len) local = pass * kCusPerXcd + len - 1 - c;
+        }
+    }
+    const int item = first + local;
+    return (local < per && item < total) ? item : -1;
+}
+
 }  // namespace chill

@@ -202,6 +202,14 @@ int chill_mask_eval(const ChillMaskDesc* mask, int32_t n, uint8_t* out);
 int chill_mask_limits(const ChillMaskDesc* mask, int32_t which, int32_t n, int32_t seq_len,
                       int32_t* out);
 
+/* The work item (tile index within the launch, longest tiles of a head first) that workgroup `workgroup` of a launch of
+ * `total` work items takes, or -1 when it has none: the XCD-contiguous order of the kernels, compiled for the host.
+ * `resident` = workgroups of the kernel that share a CU (1-3); a grid that the chip holds at once is dealt out
+ * with every second pass over an XCD's CUs in reverse.  Over the workgroups of a grid (total rounded up to a multiple
+ * of 8) the items are a permutation of 0 .. total-1.  Counterpart of the program-id -> tile arithmetic at the top of
+ * the reference's kernels (chill_fwd.py:58-61, chill_bwd.py:71-84). */
+int chill_work_item(int32_t workgroup, int32_t total, int32_t resident);
+
 /* Host twin of chill_tile_ranges_device (same functors compiled for the host). */
 int chill_tile_ranges(const ChillMaskDesc* mask, int32_t pass, int32_t T, int32_t seq_len,
                       int32_t tile_in, int32_t tile_out, int32_t* out);

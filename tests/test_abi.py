@@ -245,6 +245,32 @@ def test_tile_table():
     assert _lib.lib.chill_tile_config(0, 64, _lib.BF16, 3, out) == -8
 
 
+def test_work_items_are_a_permutation_and_resident_grids_balance():
+    """chill_work_item (the kernels' workgroup -> work item order, compiled for the host): over a grid the items are a
+    permutation of 0 .. total-1 for every grid size and every number of resident workgroups; a grid that the chip holds
+    at once gives the two (three) workgroups that share a CU items whose causal weights add up alike."""
+    f = _lib.lib.chill_work_item
+    for resident in (1, 2, 3):
+        for total in list(range(1, 530)) + [600, 767, 768, 769, 1000, 1024, 4096]:
+            grid = -(-total // 8) * 8
+            items = [f(w, total, resident) for w in range(grid)]
+            assert sorted(i for i in items if i >= 0) == list(range(total)), (resident, total)
+            if resident == 1 or total <= 256 or total > 256 * resident:
+                # one workgroup per CU, or a grid dealt out as CUs become free: XCD x takes items x * per .. in order
+                per = -(-total // 8)
+                assert all(items[w] in (-1, (w % 8) * per + w // 8) for w in range(grid)), (resident, total)
+    assert f(-1, 8, 1) == -8 and f(0, 0, 1) == -8 and f(0, 8, 0) == -8
+    # 512 workgroups, two per CU, tiles of n_tiles per head ordered longest first (weight = n_tiles - 1 - item % n_tiles):
+    # workgroups l and l + 32 of an XCD share a CU
+    for n_tiles in (16, 32, 64):
+        weight = lambda item: n_tiles - 1 - item % n_tiles
+        for xcd in range(8):
+            sums = {weight(f(8 * l + xcd, 512, 2)) + weight(f(8 * (l + 32) + xcd, 512, 2)) for l in range(32)}
+            assert sums == {n_tiles - 1}, (n_tiles, xcd, sums)
+            plain = {weight(f(8 * l + xcd, 512, 1)) + weight(f(8 * (l + 32) + xcd, 512, 1)) for l in range(32)}
+            assert len(plain) > 1
+
+
 def test_cpu_tensors_are_refused():
     import torch
 
