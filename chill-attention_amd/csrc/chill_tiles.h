@@ -268,11 +268,15 @@ constexpr int dq_stages(int mask_id, int D, int dtype, int T) {
 // workgroups per CU, not for the banded masks.  Measured on dQ alone, against dq_kernel on one box: causal B8 H16
 // T8192 2.71 / 2.90 ms, B2 H8 T8192 0.408 / 0.428, prefix-LM B4 H16 T8192 1.45 / 1.55, full mask fp16 B4 H16 T4096
 // 0.76 / 0.82; but causal B16 H16 T4096 1.63 / 1.62, B8 H8 T4096 0.509 / 0.496, B1 H8 T8192 0.227 / 0.232.
-constexpr int kDqRegs2MinSequence = 8192;
+// (from 4097 keys on, where dq_kernel leaves its 4-wave shape; full masks from 2048.  Measured on bf16 at B8 H16 since
+// the waves at a ragged end of the sequence take the complete tile's predicate-free range: causal T = 5000 / 6143 /
+// 7000 / 8000 -7.7 / -8.1 / -4.9 / -5.3 %, at T = 4096 / 3072 / 2048 against the 4-wave shape +2 / +3 / +14 %; full mask
+// T = 2048 / 3072 / 4096 / 6143 / 8000 -4 / -7 / -7 / -9.5 / -9.6 %; prefix-LM T = 5000 / 7000 -6.4 %, T = 3072 +0.5 %)
+constexpr int dq_regs2_min_sequence(int mask_id) { return mask_id == CHILL_MASK_FULL ? 2048 : 4097; }
 constexpr int kDqRegs2MinWorkgroups = 2 * 256;
 constexpr bool dq_regs2_is_optional(int D, int dtype) { return dtype != CHILL_F32 && D == 128; }
 constexpr bool dq_takes_regs2(int mask_id, long long batch_heads, int T) {
-    return !mask_is_banded(mask_id) && T >= kDqRegs2MinSequence && batch_heads * ((T + 255) / 256) >= kDqRegs2MinWorkgroups;
+    return !mask_is_banded(mask_id) && T >= dq_regs2_min_sequence(mask_id) && batch_heads * ((T + 255) / 256) >= kDqRegs2MinWorkgroups;
 }
 constexpr TileConfig dq_regs2_tile_config(int D, int dtype) {
     return TileConfig{256, 32, 4, 4 * 2 * 32 * D * elem_bytes(dtype)};

@@ -133,7 +133,7 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_FWD)["lds_bytes"] == 4 * 64 * (272 + 320)
     # short sequences and small grids at head dim 128: the 4-wave shape in forward (T <= 1024) and dQ (T <= 4096)
     for p, T, bh, waves in ((_lib.PASS_FWD, 1024, 128, 4), (_lib.PASS_FWD, 1025, 128, 8), (_lib.PASS_DQ, 4096, 128, 4),
-                            (_lib.PASS_DQ, 4097, 128, 8), (_lib.PASS_DQ, 8191, 128, 8), (_lib.PASS_FWD, 8192, 8, 8), (_lib.PASS_FWD, 8192, 16, 8),
+                            (_lib.PASS_DQ, 4097, 30, 8), (_lib.PASS_DQ, 8191, 15, 8), (_lib.PASS_FWD, 8192, 8, 8), (_lib.PASS_FWD, 8192, 16, 8),
                             (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 2048, 8, 4), (_lib.PASS_DKDV, 2048, 16, 8)):
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
@@ -174,12 +174,18 @@ def test_tile_table():
         c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=1 << 12)
         assert (c["rows"], c["waves"]) == (rows, waves), (D, c)
     assert tile_config(window, 64, torch.bfloat16, _lib.PASS_DKDV)["rows"] == 64
-    # dQ at 16-bit head dim 128 from 8192 keys on, full grids, masks that are not banded: Q and dO in registers
+    # dQ at 16-bit head dim 128 from 4097 keys on (full masks: 2048), full grids, masks that are not banded: Q and dO in
+    # registers
     regs2 = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 4 * 2 * 32 * 256}
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_DQ) == regs2
     assert tile_config(causal, 128, torch.float16, _lib.PASS_DQ, seq_len=8192, batch_heads=16) == regs2
-    for mask, T, bh in ((causal, 8191, 128), (causal, 8192, 15), (window, 16384, 128)):
+    assert tile_config(causal, 128, torch.float16, _lib.PASS_DQ, seq_len=4097, batch_heads=31) == regs2
+    assert tile_config(ca.PrefixLMChillMask(7), 128, torch.bfloat16, _lib.PASS_DQ, seq_len=6000, batch_heads=32) == regs2
+    assert tile_config(ca.FullChillMask(), 128, torch.bfloat16, _lib.PASS_DQ, seq_len=2048, batch_heads=64) == regs2
+    for mask, T, bh in ((causal, 4096, 128), (causal, 8192, 15), (causal, 4097, 30), (window, 16384, 128), (ca.FullChillMask(), 2047, 128),
+                        (ca.FullChillMask(), 2048, 63), (ca.ChunkwiseChillMask(1024, 1), 8192, 128)):
         assert tile_config(mask, 128, torch.bfloat16, _lib.PASS_DQ, seq_len=T, batch_heads=bh)["streamed"] == 64, (mask, T, bh)
+    assert tile_config(causal, 64, torch.bfloat16, _lib.PASS_DQ, seq_len=8192, batch_heads=128)["streamed"] == 64
     # dK/dV at 16-bit head dim 128: K in registers, two 32-key blocks per wave (256 key rows, 4 waves, 32-row tiles in
     # four stages) for long sequences on a grid of two workgroups per CU, except under banded masks; else the paired kernel
     regs = {"rows": 256, "streamed": 32, "waves": 4, "lds_bytes": 256 * 256 + 4 * (2 * 32 * 256 + 2 * 32 * 4)}

@@ -534,7 +534,8 @@ DKDV_REGS_CASES = [
     ("full-lens-f16", torch.float16, 2, 16, 16, 4130, ("FullChillMask", ()), (4130, 3000)),
     ("prefix-lm", torch.bfloat16, 2, 16, 16, 4096, ("PrefixLMChillMask", (1024,)), None),
     ("prefix-lm-gqa-ragged", torch.float16, 1, 64, 32, 4111, ("PrefixLMChillMask", (77,)), (4001,)),
-    # sequences from 8192 on: dQ takes its register-resident kernel (chill_bwd_dq_gen.h, gen_dq_loop.py) as well
+    # longer sequences (dQ takes its register-resident kernel, chill_bwd_dq_gen.h and gen_dq_loop.py, from 4097 keys on, under a
+    # full mask from 2048, on grids of at least 512 workgroups)
     ("long-causal", torch.bfloat16, 1, 16, 16, 8192, ("CausalChillMask", ()), None),
     ("long-causal-gqa-lens-f16", torch.float16, 2, 16, 8, 8192, ("CausalChillMask", ()), (8192, 5000)),
     ("long-full-ragged", torch.bfloat16, 1, 32, 16, 8200, ("FullChillMask", ()), None),
@@ -688,10 +689,11 @@ def test_dkdv_with_resident_keys_and_generated_loop(case):
     mask = make_mask(m)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DKDV, seq_len=T, batch_heads=B * Hkv)
     assert (cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32), f"served by {cfg}"
-    # (dQ has such a kernel too, for sequences from 8192 on: the cases of that length below)
+    # (dQ has such a kernel too, for sequences from 4097 keys on, full masks from 2048)
     cfg = tile_config(mask, D, dtype, _lib.PASS_DQ, seq_len=T, batch_heads=B * H)
     banded = m[0] in ("ChunkwiseChillMask", "SlidingWindowChillMask")
-    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == (T >= 8192 and not banded and D == 128), f"dQ served by {cfg}"
+    dq_regs = (not banded and D == 128 and T >= (2048 if m[0] == "FullChillMask" else 4097) and B * H * -(-T // 256) >= 512)
+    assert ((cfg["rows"], cfg["waves"], cfg["streamed"]) == (256, 4, 32)) == dq_regs, f"dQ served by {cfg}"
     torch.manual_seed(stable_seed(case[0]))
     q, k, v = (make_qkv((B, h, T, D), dtype, False).requires_grad_() for h in (H, Hkv, Hkv))
     lens_t = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
