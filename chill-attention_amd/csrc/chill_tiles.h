@@ -352,7 +352,16 @@ constexpr int dkdv_regs_stages(int D) { return D == 256 ? 2 : 4; }
 // quarter of the size and fill a small grid better: B2 H16 T4096 (512 workgroups of this kernel) causal 0.20 / 0.17,
 // prefix-LM 0.20 / 0.18 (but full mask 0.28 / 0.38); B4 H16 T4096 (1024) causal 0.37 / 0.38: from four workgroups per CU on.
 constexpr int kDkdvRegsBlocks128 = 2;
-constexpr int kDkdvRegsMinSequence = 4096;
+// Sequence lengths from which it is taken, by what the mask leaves of a key block's loop (measured against the other
+// kernel on bf16 grids of 1024 .. 4096 workgroups, B8 .. B32 H16): under a full mask every tile is predicate-free and it
+// wins from the shortest sequences tried (T = 1024 / 2048 / 3072 / 4000: -16 / -17 / -18 / -17 % at head dim 128, -21 / -27 /
+// -27 / -23 % at head dim 64); under a causal mask the first tiles of a key block run outside the generated loop and the
+// runs shrink with the sequence (head dim 128: T = 1024 / 2048 / 3072 / 3500 / 4000 +14 / +1 / -3 / -4.5 / -5 .. -8 %;
+// head dim 64: T = 2048 / 3072 / 3500 / 4000 +5 .. +17 / -2 .. +1.5 / -5 / -3 .. -5 %); prefix-LM lies between the two
+// (prefix 512, head dim 128: -6 .. -10 % from T = 1024 on) and takes the causal limits; the banded masks it serves keep 4096.
+constexpr int dkdv_regs_min_sequence(int mask_id, int D) {
+    return mask_id == CHILL_MASK_FULL ? 1024 : mask_is_banded(mask_id) ? 4096 : D >= 128 ? 3072 : 3500;
+}
 constexpr int kDkdvRegsMinWorkgroups = 2 * 256;
 constexpr int kDkdvRegsMinWorkgroups64 = 4 * 256;
 constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && (D == 128 || D == 64); }
@@ -369,7 +378,7 @@ constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0, long long
            (mask_id == CHILL_MASK_SLIDING_WINDOW && band_keys >= kDkdvRegsWideBand);
 }
 constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, long long band_keys, int D, long long batch_kv_heads, int T) {
-    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, band_keys, D)) && T >= kDkdvRegsMinSequence &&
+    return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, band_keys, D)) && T >= dkdv_regs_min_sequence(mask_id, D) &&
            batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >=
                (D >= 128 ? kDkdvRegsMinWorkgroups : kDkdvRegsMinWorkgroups64);
 }

@@ -170,7 +170,7 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.float32, _lib.PASS_FWD, seq_len=1024, batch_heads=9)["lds_bytes"] == 4 * (2 * 32 * 512 + 512)
     # dK/dV at 16-bit head dims <= 64: 64 key rows per workgroup of 4 waves, several workgroups per CU (at head dim 64
     # for short sequences, small grids and banded masks; long sequences: K in registers, below)
-    for D, T, rows, waves in ((64, 4095, 64, 4), (32, None, 64, 4), (32, 8192, 64, 4)):
+    for D, T, rows, waves in ((64, 3499, 64, 4), (32, None, 64, 4), (32, 8192, 64, 4)):
         c = tile_config(causal, D, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=1 << 12)
         assert (c["rows"], c["waves"]) == (rows, waves), (D, c)
     assert tile_config(window, 64, torch.bfloat16, _lib.PASS_DKDV)["rows"] == 64
@@ -192,7 +192,12 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.bfloat16, _lib.PASS_DKDV) == regs
     assert tile_config(causal, 128, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs
     assert tile_config(causal, 128, torch.float16, _lib.PASS_DKDV, seq_len=4096, batch_heads=32) == regs
-    for mask, T, bh in ((causal, 4095, 128), (causal, 4096, 31), (window, 8192, 128), (window, None, 1 << 20)):
+    # (from 3072 keys on under causal-like masks, 3500 at head dim 64; under a full mask from 1024)
+    assert tile_config(causal, 128, torch.float16, _lib.PASS_DKDV, seq_len=3072, batch_heads=64) == regs
+    assert tile_config(ca.PrefixLMChillMask(9), 128, torch.float16, _lib.PASS_DKDV, seq_len=3500, batch_heads=64) == regs
+    assert tile_config(ca.FullChillMask(), 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=1024, batch_heads=128) == regs
+    for mask, T, bh in ((causal, 3071, 128), (causal, 4096, 31), (window, 8192, 128), (window, None, 1 << 20), (ca.FullChillMask(), 1023, 256),
+                        (ca.FullChillMask(), 1024, 127), (ca.ChunkwiseChillMask(128, 2), 4095, 128)):
         c = tile_config(mask, 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
         assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
     # chunkwise masks whose chunks are a multiple of a wave's 64 key rows (no partly masked block inside the band) take
@@ -234,6 +239,8 @@ def test_tile_table():
     assert tile_config(ca.PrefixLMChillMask(1024), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     assert tile_config(ca.ChunkwiseChillMask(512, 1), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     assert tile_config(causal, 64, torch.float16, _lib.PASS_DKDV, seq_len=4096, batch_heads=64) == regs64
+    assert tile_config(causal, 64, torch.float16, _lib.PASS_DKDV, seq_len=3500, batch_heads=74) == regs64
+    assert tile_config(ca.FullChillMask(), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=1024, batch_heads=256) == regs64
     assert tile_config(ca.SlidingWindowChillMask(4096, 100), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     for mask, T, bh in ((causal, 4096, 63), (causal, 8192, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64),
                         (ca.ChunkwiseChillMask(256, 1), 8192, 128), (window, 8192, 128)):

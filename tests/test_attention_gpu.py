@@ -546,6 +546,11 @@ DKDV_REGS_CASES = [
     ("chunkwise-64x4-gqa-lens", torch.bfloat16, 4, 16, 8, 4096, ("ChunkwiseChillMask", (64, 4)), (4096, 3000, 77, 4001)),
     ("chunkwise-1024x1-ragged-f16", torch.float16, 1, 32, 32, 4140, ("ChunkwiseChillMask", (1024, 1)), None),
     ("chunkwise-192x0", torch.bfloat16, 1, 32, 32, 4096, ("ChunkwiseChillMask", (192, 0)), None),
+    # shorter sequences: from 1024 keys on under a full mask, from 3072 under causal-like masks
+    ("full-T1024-gqa-lens", torch.bfloat16, 16, 16, 8, 1024, ("FullChillMask", ()), (1024, 1000, 5, 513, 1024, 1, 256, 257, 1023, 700, 64, 1024, 33, 900, 512, 1024)),
+    ("full-T1100-ragged-f16", torch.float16, 8, 16, 16, 1100, ("FullChillMask", ()), None),
+    ("causal-T3072", torch.bfloat16, 3, 16, 16, 3072, ("CausalChillMask", ()), None),
+    ("prefix-lm-T3300-gqa-ragged-lens-f16", torch.float16, 6, 16, 8, 3300, ("PrefixLMChillMask", (100,)), (3300, 3000, 3299, 77, 1700, 3300)),
     # sliding windows of 4096 keys and more: a long loop again, with masked tiles at both ends of a wave's run
     ("sliding-4096+0", torch.bfloat16, 2, 16, 16, 8192, ("SlidingWindowChillMask", (4096, 0)), None),
     ("sliding-3000+2000-gqa-ragged-lens-f16", torch.float16, 1, 32, 16, 8200, ("SlidingWindowChillMask", (3000, 2000)), (8100,)),
@@ -562,6 +567,8 @@ DKDV_REGS_CASES_64 = [
     ("long-prefix-lm", torch.bfloat16, 1, 32, 32, 8192, ("PrefixLMChillMask", (1024,)), None),
     ("chunkwise-512x1-f16", torch.float16, 2, 32, 16, 8192, ("ChunkwiseChillMask", (512, 1)), (8000, 8192)),
     ("sliding-4096+100", torch.bfloat16, 2, 32, 32, 8192, ("SlidingWindowChillMask", (4096, 100)), None),
+    ("full-T1024", torch.bfloat16, 16, 16, 16, 1024, ("FullChillMask", ()), None),
+    ("causal-T3500-gqa-f16", torch.float16, 10, 16, 8, 3500, ("CausalChillMask", ()), None),
 ]
 
 
