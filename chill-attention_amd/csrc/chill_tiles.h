@@ -364,6 +364,14 @@ constexpr int dkdv_regs_min_sequence(int mask_id, int D) {
 }
 constexpr int kDkdvRegsMinWorkgroups = 2 * 256;
 constexpr int kDkdvRegsMinWorkgroups64 = 4 * 256;
+// (by mask as well: under a full mask it wins on one workgroup per CU already, B1 H16 T4096 -24 % at head dim 128 and -38 %
+// at head dim 64, where causal and prefix-LM masks lose 10-19 %; at head dim 64 the causal-like masks win on 512 workgroups
+// from 8192 keys on, B1 H16 T8192 -13 %, B1 H8 T16384 -15 %, and lose 4-9 % at T = 4096)
+constexpr long long dkdv_regs_min_workgroups(int mask_id, int D, int T) {
+    if (mask_id == CHILL_MASK_FULL) return 256;
+    if (D >= 128) return kDkdvRegsMinWorkgroups;
+    return (!mask_is_banded(mask_id) && T >= 8192) ? kDkdvRegsMinWorkgroups64 / 2 : kDkdvRegsMinWorkgroups64;
+}
 constexpr bool dkdv_regs_is_optional(int D, int dtype) { return dtype != CHILL_F32 && (D == 128 || D == 64); }
 // Banded masks take it only when a wave's 64 key rows lie in one chunk, so that its tiles are all predicate-free
 // and all alike: chunkwise masks whose chunk size is a multiple of 64 (`mask_arg0` = the mask's first argument;
@@ -379,8 +387,7 @@ constexpr bool dkdv_regs_serves_band(int mask_id, long long mask_arg0, long long
 }
 constexpr bool dkdv_takes_regs(int mask_id, long long mask_arg0, long long band_keys, int D, long long batch_kv_heads, int T) {
     return (!mask_is_banded(mask_id) || dkdv_regs_serves_band(mask_id, mask_arg0, band_keys, D)) && T >= dkdv_regs_min_sequence(mask_id, D) &&
-           batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >=
-               (D >= 128 ? kDkdvRegsMinWorkgroups : kDkdvRegsMinWorkgroups64);
+           batch_kv_heads * ((T + 128 * kDkdvRegsBlocks128 - 1) / (128 * kDkdvRegsBlocks128)) >= dkdv_regs_min_workgroups(mask_id, D, T);
 }
 
 // `regs`: the row of dkdv_regs_kernel where that kernel is an option (dkdv_regs_is_optional)

@@ -196,8 +196,9 @@ def test_tile_table():
     assert tile_config(causal, 128, torch.float16, _lib.PASS_DKDV, seq_len=3072, batch_heads=64) == regs
     assert tile_config(ca.PrefixLMChillMask(9), 128, torch.float16, _lib.PASS_DKDV, seq_len=3500, batch_heads=64) == regs
     assert tile_config(ca.FullChillMask(), 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=1024, batch_heads=128) == regs
+    assert tile_config(ca.FullChillMask(), 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=4096, batch_heads=16) == regs
     for mask, T, bh in ((causal, 3071, 128), (causal, 4096, 31), (window, 8192, 128), (window, None, 1 << 20), (ca.FullChillMask(), 1023, 256),
-                        (ca.FullChillMask(), 1024, 127), (ca.ChunkwiseChillMask(128, 2), 4095, 128)):
+                        (ca.FullChillMask(), 1024, 63), (ca.FullChillMask(), 4096, 15), (ca.ChunkwiseChillMask(128, 2), 4095, 128)):
         c = tile_config(mask, 128, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
         assert (c["rows"], c["waves"], c["streamed"]) == (128, 8, 64), (mask, T, bh, c)
     # chunkwise masks whose chunks are a multiple of a wave's 64 key rows (no partly masked block inside the band) take
@@ -240,9 +241,11 @@ def test_tile_table():
     assert tile_config(ca.ChunkwiseChillMask(512, 1), 64, torch.float16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
     assert tile_config(causal, 64, torch.float16, _lib.PASS_DKDV, seq_len=4096, batch_heads=64) == regs64
     assert tile_config(causal, 64, torch.float16, _lib.PASS_DKDV, seq_len=3500, batch_heads=74) == regs64
-    assert tile_config(ca.FullChillMask(), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=1024, batch_heads=256) == regs64
+    assert tile_config(ca.FullChillMask(), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=1024, batch_heads=64) == regs64
+    assert tile_config(causal, 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=8192, batch_heads=16) == regs64
+    assert tile_config(ca.PrefixLMChillMask(5), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=16384, batch_heads=8) == regs64
     assert tile_config(ca.SlidingWindowChillMask(4096, 100), 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=8192, batch_heads=128) == regs64
-    for mask, T, bh in ((causal, 4096, 63), (causal, 8192, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64),
+    for mask, T, bh in ((causal, 4096, 63), (causal, 8192, 15), (causal, 8191, 31), (ca.ChunkwiseChillMask(512, 1), 8192, 31), (ca.ChunkwiseChillMask(128, 2), 16384, 64),
                         (ca.ChunkwiseChillMask(256, 1), 8192, 128), (window, 8192, 128)):
         c = tile_config(mask, 64, torch.bfloat16, _lib.PASS_DKDV, seq_len=T, batch_heads=bh)
         assert (c["rows"], c["waves"], c["streamed"]) == (64, 4, 64), (mask, T, bh, c)

@@ -550,6 +550,8 @@ DKDV_REGS_CASES = [
     ("full-T1024-gqa-lens", torch.bfloat16, 16, 16, 8, 1024, ("FullChillMask", ()), (1024, 1000, 5, 513, 1024, 1, 256, 257, 1023, 700, 64, 1024, 33, 900, 512, 1024)),
     ("full-T1100-ragged-f16", torch.float16, 8, 16, 16, 1100, ("FullChillMask", ()), None),
     ("causal-T3072", torch.bfloat16, 3, 16, 16, 3072, ("CausalChillMask", ()), None),
+    # (one workgroup per CU under a full mask)
+    ("full-256-workgroups-gqa-f16", torch.float16, 1, 32, 16, 4100, ("FullChillMask", ()), (4001,)),
     ("prefix-lm-T3300-gqa-ragged-lens-f16", torch.float16, 6, 16, 8, 3300, ("PrefixLMChillMask", (100,)), (3300, 3000, 3299, 77, 1700, 3300)),
     # sliding windows of 4096 keys and more: a long loop again, with masked tiles at both ends of a wave's run
     ("sliding-4096+0", torch.bfloat16, 2, 16, 16, 8192, ("SlidingWindowChillMask", (4096, 0)), None),
@@ -568,6 +570,8 @@ DKDV_REGS_CASES_64 = [
     ("chunkwise-512x1-f16", torch.float16, 2, 32, 16, 8192, ("ChunkwiseChillMask", (512, 1)), (8000, 8192)),
     ("sliding-4096+100", torch.bfloat16, 2, 32, 32, 8192, ("SlidingWindowChillMask", (4096, 100)), None),
     ("full-T1024", torch.bfloat16, 16, 16, 16, 1024, ("FullChillMask", ()), None),
+    ("full-256-workgroups", torch.bfloat16, 1, 16, 16, 4096, ("FullChillMask", ()), None),
+    ("causal-512-workgroups-T8192-gqa", torch.bfloat16, 1, 32, 16, 8192, ("CausalChillMask", ()), (8100,)),
     ("causal-T3500-gqa-f16", torch.float16, 10, 16, 8, 3500, ("CausalChillMask", ()), None),
 ]
 
