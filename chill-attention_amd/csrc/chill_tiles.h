@@ -82,6 +82,7 @@ constexpr long long kNarrowBand = 1;
 // the neighbouring kernels more than it gains).  T = kLongSequence selects the long-sequence row.
 constexpr int kLongSequence = 0x7fffffff;
 constexpr int kFwdShortSequence = 1024;
+constexpr int kFwdShortSequenceFull = 768;
 constexpr int kDqShortSequence = 4096;
 // The same shape is taken when the 8-wave one would leave CUs without a workgroup (B1 H8 T8192 causal:
 // forward -7 %, dQ -17 %; with twice as many heads the 8-wave shape wins again).
@@ -94,7 +95,10 @@ constexpr int kComputeUnits = 256;
 constexpr int kFwdWideBand = 1024;
 constexpr bool fwd_takes_short_row(int mask_id, long long band_keys, long long batch_heads, int T) {
     (void)batch_heads;
-    return T <= kFwdShortSequence || (mask_is_banded(mask_id) && band_keys < kFwdWideBand);
+    // (under a full mask the 8-wave shape, whose loop is predicate-free from its first tile on, wins from 769 keys on:
+    // B16 H16 T = 1024 / 1000 -12 / -7 %, T = 768 / 512 +2 / -1 %; causal T = 1024 / 768 / 512 +3 / +41 / +23 %)
+    return T <= (mask_id == CHILL_MASK_FULL ? kFwdShortSequenceFull : kFwdShortSequence) ||
+           (mask_is_banded(mask_id) && band_keys < kFwdWideBand);
 }
 constexpr bool dq_takes_short_row(long long batch_heads, int T) {
     return T <= kDqShortSequence || batch_heads * ((T + 255) / 256) <= kComputeUnits;

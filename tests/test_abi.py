@@ -136,6 +136,9 @@ def test_tile_table():
                             (_lib.PASS_DQ, 4097, 30, 8), (_lib.PASS_DQ, 8191, 15, 8), (_lib.PASS_FWD, 8192, 8, 8), (_lib.PASS_FWD, 8192, 16, 8),
                             (_lib.PASS_DQ, 8192, 8, 4), (_lib.PASS_DKDV, 2048, 8, 4), (_lib.PASS_DKDV, 2048, 16, 8)):
         assert tile_config(causal, 128, torch.bfloat16, p, seq_len=T, batch_heads=bh)["waves"] == waves, (p, T, bh)
+    # (under a full mask the forward takes its 8-wave shape from 769 keys on)
+    assert tile_config(ca.FullChillMask(), 128, torch.bfloat16, _lib.PASS_FWD, seq_len=768, batch_heads=128)["waves"] == 4
+    assert tile_config(ca.FullChillMask(), 128, torch.bfloat16, _lib.PASS_FWD, seq_len=769, batch_heads=128)["waves"] == 8
     assert tile_config(causal, 128, torch.float32, _lib.PASS_DQ, seq_len=128) == tile_config(causal, 128, torch.float32, _lib.PASS_DQ)
     assert _lib.lib.chill_tile_config_for_shape(1, 128, _lib.BF16, 0, 1, 0, (ctypes.c_int32 * 4)()) == -8
     # launches far too small for the chip: 32 rows per workgroup; fp32 much further up than 16-bit inputs, and furthest

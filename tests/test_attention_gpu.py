@@ -427,8 +427,8 @@ RAMP_CASES = [
     ("d64-loop-f16", torch.float16, 64, 3, 8, 4, 1024, (128, 4), (0, 1, 4), "all", None),
     ("d64-loop-paired-second-only", torch.float16, 64, 8, 16, 16, 2048, (128, 4), (0, 1, 7), "low", None),
     ("d64-loop-paired-lens", torch.bfloat16, 64, 8, 16, 16, 2048, (128, 4), (1, 7), "wave", (2048, 3, 999, 1024, 2048, 1500, 64, 129)),
-    ("d128-short-row", torch.bfloat16, 128, 8, 8, 8, 1024, (128, 4), (0, 1), "all", None),
-    ("d128-short-row-f16", torch.float16, 128, 8, 8, 8, 1024, (128, 4), (0, 1, 4), "wave", None),
+    ("d128-short-row", torch.bfloat16, 128, 8, 8, 8, 768, (128, 4), (0, 1), "all", None),
+    ("d128-short-row-f16", torch.float16, 128, 8, 8, 8, 1024, (128, 4), (1, 4), "wave", None),
     ("d32", torch.float16, 32, 3, 8, 8, 1024, (128, 4), (0, 1), "all", None),
     ("d32-bf16", torch.bfloat16, 32, 3, 8, 8, 1024, (128, 4), (0, 1), "all", None),
     ("d256-regs", torch.bfloat16, 256, 2, 8, 8, 2048, (128, 4), (0, 1), "all", None),
