@@ -39,9 +39,9 @@ PEAK_HBM_GBS = 8000.0
 # sources it was measured on (kernel_sources_digest below); with other sources the line reports null.
 TRAFFIC_SOURCE = "profiles/c3_causal_bf16_fwd_bwd_kernels.md"
 MEASURED_TRAFFIC = {
-    ("C3", "chill_fwd"): (593745 * 2.0 + 344065) * 1024,
-    ("C3", "chill_bwd_dq_delta"): (923530 * 2.0 + 290372) * 1024,
-    ("C3", "chill_bwd_dkdv"): (829643 * 2.0 + 577536) * 1024,
+    ("C3", "chill_fwd"): (594702 * 2.0 + 344064) * 1024,
+    ("C3", "chill_bwd_dq_delta"): (924862 * 2.0 + 290374) * 1024,
+    ("C3", "chill_bwd_dkdv"): (830308 * 2.0 + 577536) * 1024,
 }
 
 
